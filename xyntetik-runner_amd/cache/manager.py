@@ -63,6 +63,10 @@ def pages_for_spec(spec: KVSpec, page_size: int, max_tokens: int, max_requests: 
     are all held until the portion is cached.
     """
     full = max(1, -(-int(max_tokens) // page_size))
+    if spec.stride > 1:
+        # one entry for every `stride` positions: what the tokens' pages would hold, thinned out,
+        # and for every request the page it has begun
+        return -(-full // spec.stride) + max_requests
     if spec.window is None or max_step_tokens is None:
         return full
     per_request = -(-spec.window // page_size) + 2
@@ -100,7 +104,7 @@ class CacheManager:
     def capacity_tokens(self) -> int:
         """The most tokens one request can hold: what the smallest pool of a group that keeps every
         key holds.  A group that keeps a window gives pages back as a request grows and sets no limit."""
-        full = [g.pool.size * self.page_size for g in self.groups if g.spec.window is None]
+        full = [g.pool.size * self.page_size * g.spec.stride for g in self.groups if g.spec.window is None]
         return min(full) if full else 1 << 62
 
     def max_portion(self) -> int:
@@ -114,7 +118,11 @@ class CacheManager:
                 best = min(best, max(1, (g.pool.size - behind) * self.page_size))
         return best
 
-    def pages_for(self, n_tokens: int) -> int:
+    def pages_for(self, n_tokens: int, group: Optional[int] = None) -> int:
+        """Pages that ``n_tokens`` positions fill (in ``group``: a group with a stride holds one entry
+        for every ``stride`` positions that are complete)."""
+        if group is not None:
+            n_tokens = n_tokens // self.groups[group].spec.stride
         return -(-n_tokens // self.page_size)
 
     def free_pages(self, group: int = 0) -> int:
@@ -133,15 +141,15 @@ class CacheManager:
         return self.slots.n_free > 0
 
     def _new_pages_needed(self, rc: RequestCache, new_len: int) -> List[int]:
-        want = self.pages_for(new_len)
-        for t in rc.tables:
-            if len(t) < want:
+        for gi, t in enumerate(rc.tables):
+            if len(t) < self.pages_for(new_len, gi):
                 break
         else:
             return self._no_pages           # the usual case of a decoded token (callers only read it)
         need = []
         for gi, g in enumerate(self.groups):
             have = len(rc.tables[gi])
+            want = self.pages_for(new_len, gi)
             # pages wholly below the window of the first new query are never read or written
             lo_page = first_needed_position(rc.n_tokens, g.spec.window) // self.page_size
             need.append(sum(1 for i in range(have, want) if i >= lo_page))
@@ -162,15 +170,15 @@ class CacheManager:
     def pages_needed_new(self, new_len: int) -> List[int]:
         """Pages per group that a request not yet admitted needs for its first ``new_len`` tokens
         (all of them: a window gives pages back only once the tokens are cached)."""
-        return [self.pages_for(new_len)] * len(self.groups)
+        return [self.pages_for(new_len, gi) for gi in range(len(self.groups))]
 
     def trim(self, req_id: Hashable) -> None:
         """Give back the pages reserved beyond the tokens the request holds (for a step that
         reserved and then did not run)."""
         rc = self.requests[req_id]
-        keep = self.pages_for(rc.n_tokens)
         for gi, g in enumerate(self.groups):
             table = rc.tables[gi]
+            keep = self.pages_for(rc.n_tokens, gi)
             while len(table) > keep:
                 page = table.pop()
                 rc.version += 1             # who copied the table must not take its length for its contents
@@ -192,13 +200,13 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             table = rc.tables[gi]
             lo_page = first_needed_position(rc.n_tokens, g.spec.window) // self.page_size
-            for i in range(len(table), self.pages_for(new_len)):
+            for i in range(len(table), self.pages_for(new_len, gi)):
                 table.append(g.pool.take() if i >= lo_page else -1)
 
     def advance(self, req_id: Hashable, new_len: int) -> None:
         """Positions below ``new_len`` are now cached; give back pages a window has passed."""
         rc = self.requests[req_id]
-        if self.pages_for(new_len) > min((len(t) for t in rc.tables), default=self.pages_for(new_len)):
+        if any(self.pages_for(new_len, gi) > len(t) for gi, t in enumerate(rc.tables)):
             raise ValueError(f"request {req_id!r}: {new_len} tokens were not reserved")
         rc.n_tokens = new_len
         rc.fresh = False
@@ -245,6 +253,6 @@ class CacheManager:
         for rc in self.requests.values():
             for gi, g in enumerate(self.groups):
                 lo = first_needed_position(rc.n_tokens, g.spec.window)
-                for pos in range(lo, rc.n_tokens):
+                for pos in range(lo, rc.n_tokens // g.spec.stride):
                     if rc.tables[gi][pos // self.page_size] < 0:
                         raise AssertionError(f"request {rc.req_id!r}: position {pos} of group {gi} has no page")

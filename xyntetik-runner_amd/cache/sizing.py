@@ -22,19 +22,29 @@ def cache_groups(kv_specs: Sequence[Optional[KVSpec]], cache_of: Sequence[Option
     (entries that read another entry's cache add nothing)."""
     specs: List[KVSpec] = []
     owners: List[int] = []
-    for kv, of in zip(kv_specs, cache_of):
-        if kv is None or of is not None:
-            continue
-        if kv not in specs:
-            specs.append(kv)
+
+    def count(spec: KVSpec) -> None:
+        if spec not in specs:
+            specs.append(spec)
             owners.append(0)
-        owners[specs.index(kv)] += 1
+        owners[specs.index(spec)] += 1
+
+    # in the order `CacheStorage` meets them: an entry's own group, then the group of its block means
+    for i, (kv, of) in enumerate(zip(kv_specs, cache_of)):
+        if kv is None:
+            continue
+        if of is None:
+            count(kv)
+            if kv.pooled:
+                count(kv.pooled_spec())
+        elif kv.pooled and (kv_specs[of] is None or kv_specs[of].pooled != kv.pooled):
+            count(kv.pooled_spec())         # a reader whose blocks differ from the owner's keeps its own means
     return specs, owners
 
 
 def page_bytes(spec: KVSpec, n_layers: int, page_size: int, element_size: int) -> int:
     """Bytes of one page number of a group: keys and values of all its layers."""
-    return 2 * n_layers * spec.num_kv_heads * spec.head_dim * page_size * element_size
+    return n_layers * spec.num_kv_heads * (spec.head_dim + spec.value_dim) * page_size * element_size
 
 
 def size_pools(specs: Sequence[KVSpec], owners: Sequence[int], page_size: int, element_size: int,
@@ -58,19 +68,23 @@ def size_pools(specs: Sequence[KVSpec], owners: Sequence[int], page_size: int, e
     sizes: List[Optional[int]] = []
     left = int(budget_bytes)
     for s, b in zip(specs, bpp):
-        if s.window is None:
+        if s.stride > 1:
+            n = pages_for_spec(s, page_size, max_requests * int(max_model_len), max_requests, step)
+            sizes.append(n)
+            left -= (n + 1) * b
+        elif s.window is None:
             sizes.append(None)
             left -= b                                           # the null page
         else:
             n = pages_for_spec(s, page_size, max_requests * int(max_model_len), max_requests, step)
             sizes.append(n)
             left -= (n + 1) * b
-    per_page = sum(b for s, b in zip(specs, bpp) if s.window is None)
+    per_page = sum(b for s, b in zip(specs, bpp) if s.window is None and s.stride == 1)
     pages = want * max_requests
     if per_page:
         pages = min(pages, left // per_page if left > 0 else 0)
     if left < 0 or (per_page and pages < want):
-        need = sum(((want if s.window is None else n) + 1) * b for s, b, n in zip(specs, bpp, sizes))
+        need = sum(((want if n is None else n) + 1) * b for s, b, n in zip(specs, bpp, sizes))
         raise CacheTooSmall(
             f"the cache does not hold one request of {max_model_len} tokens: that takes {need / 2**30:.2f} GiB, "
             f"{max(0, int(budget_bytes)) / 2**30:.2f} GiB are left after the weights; "

@@ -3,14 +3,15 @@
 For every entry of the run order that owns a cache: keys ``[pages, Hk, page_size, D]``
 and values ``[pages, Hk, D, page_size]`` (values transposed inside a page so that
 attention reads several positions of one channel with one load), in the engine's
-dtype.  For every entry whose mixer has state of fixed size: ``[slots + 1, *shape]``; row
-``null_slot`` (the last) belongs to no request.
+dtype.  A layer that keeps block means (``KVSpec.pooled``) has a second pair of tensors of the
+same layout in the group of its blocks.  For every tensor of fixed-size state a layer names:
+``[slots + 1, *shape]``; row ``null_slot`` (the last) belongs to no request.
 Page 0 is the null page.  Nothing is zeroed when a page changes hands: reads are
 bounded by a request's length, so a page's old contents are never seen.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Union
 
 import torch
@@ -26,7 +27,12 @@ class LayerCache:
     owns: bool                 # this entry writes keys and values (False: it reads another entry's)
     k: Optional[torch.Tensor]
     v: Optional[torch.Tensor]
-    state: Optional[torch.Tensor] = None    # [slots + 1, *shape]; the last row is nobody's
+    state: Optional[torch.Tensor] = None    # [slots + 1, *shape]; the last row is nobody's (the mixer's own, if it has one)
+    states: Dict[str, torch.Tensor] = field(default_factory=dict)     # every state tensor of the layer by name
+    pool_group: int = -1                    # the block table of the block means, for a layer that keeps them
+    pool_k: Optional[torch.Tensor] = None   # [pages, Hk, page_size, D]: entry b of a request is block b's mean key
+    pool_v: Optional[torch.Tensor] = None   # [pages, Hk, Dv, page_size]
+    pool_owns: bool = False                 # this entry writes the block means (False: another entry's are the same)
 
 
 class CacheStorage:
@@ -43,13 +49,32 @@ class CacheStorage:
         self.group_specs: List[KVSpec] = []
         self.group_pages: List[int] = []        # usable pages of each group (the null page comes on top)
         self.layers: List[LayerCache] = []
+
+        def group_of(spec: KVSpec) -> int:
+            if spec not in self.group_specs:
+                self.group_specs.append(spec)
+                self.group_pages.append(max(1, int(sized(spec))))
+            return self.group_specs.index(spec)
+
+        def pages_of(spec: KVSpec):
+            n_pages = self.group_pages[group_of(spec)] + 1
+            return (torch.zeros((n_pages, spec.num_kv_heads, page_size, spec.head_dim), dtype=dtype, device=device),
+                    torch.zeros((n_pages, spec.num_kv_heads, spec.value_dim, page_size), dtype=dtype, device=device))
+
+        def states_of(st) -> Dict[str, torch.Tensor]:
+            # one row more than requests: the last is nobody's (rows that pad a recorded step use it)
+            named = {} if st is None else ({"mixer": st} if isinstance(st, StateSpec) else dict(st))
+            return {name: torch.zeros((n_slots + 1,) + tuple(s.shape), dtype=s.dtype or dtype, device=device)
+                    for name, s in named.items()}
+
         for i, (kv, st) in enumerate(zip(kv_specs, state_specs)):
             owner = cache_of[i]
+            states = states_of(st)
             if owner is not None:
                 src = self.layers[owner]
                 if kv is not None and src.k is not None:
                     okv = kv_specs[owner]
-                    if (okv.num_kv_heads, okv.head_dim) != (kv.num_kv_heads, kv.head_dim):
+                    if (okv.num_kv_heads, okv.head_dim, okv.value_dim) != (kv.num_kv_heads, kv.head_dim, kv.value_dim):
                         raise ValueError(f"run order entry {i} reads the cache of entry {owner}, "
                                          f"whose heads or head size differ")
                     # the owner's window decides which pages exist: a reader that looks further
@@ -57,26 +82,32 @@ class CacheStorage:
                     if okv.window is not None and (kv.window is None or kv.window > okv.window):
                         raise ValueError(f"run order entry {i} (window {kv.window}) reads the cache of entry {owner}, "
                                          f"which keeps only the last {okv.window} keys")
-                self.layers.append(LayerCache(src.group, page_size, False, src.k, src.v, None))
+                lc = LayerCache(src.group, page_size, False, src.k, src.v, states.get("mixer"), states)
+                if kv is not None and kv.pooled:
+                    # block means of the owner's keys: the owner's own where its blocks are as long,
+                    # else a cache of this entry's making
+                    if src.pool_k is not None and kv_specs[owner].pooled == kv.pooled:
+                        lc.pool_group, lc.pool_k, lc.pool_v = src.pool_group, src.pool_k, src.pool_v
+                    else:
+                        ps = kv.pooled_spec()
+                        lc.pool_group, lc.pool_owns = group_of(ps), True
+                        lc.pool_k, lc.pool_v = pages_of(ps)
+                self.layers.append(lc)
                 continue
             group, k, v = -1, None, None
             if kv is not None:
-                if kv not in self.group_specs:
-                    self.group_specs.append(kv)
-                    self.group_pages.append(max(1, int(sized(kv))))
-                group = self.group_specs.index(kv)
-                n_pages = self.group_pages[group] + 1
-                k = torch.zeros((n_pages, kv.num_kv_heads, page_size, kv.head_dim), dtype=dtype, device=device)
-                v = torch.zeros((n_pages, kv.num_kv_heads, kv.head_dim, page_size), dtype=dtype, device=device)
-            state = None
-            if st is not None:
-                # one row more than requests: the last is nobody's (rows that pad a recorded step use it)
-                state = torch.zeros((n_slots + 1,) + tuple(st.shape), dtype=st.dtype, device=device)
-            self.layers.append(LayerCache(group, page_size, True, k, v, state))
+                group = group_of(kv)
+                k, v = pages_of(kv)
+            lc = LayerCache(group, page_size, True, k, v, states.get("mixer"), states)
+            if kv is not None and kv.pooled:
+                ps = kv.pooled_spec()
+                lc.pool_group, lc.pool_owns = group_of(ps), True
+                lc.pool_k, lc.pool_v = pages_of(ps)
+            self.layers.append(lc)
 
     def bytes_per_token(self) -> int:
         total = 0
         for lc in self.layers:
             if lc.owns and lc.k is not None:
-                total += 2 * lc.k.shape[1] * lc.k.shape[3] * lc.k.element_size()
+                total += lc.k.shape[1] * (lc.k.shape[3] + lc.v.shape[2]) * lc.k.element_size()
         return total

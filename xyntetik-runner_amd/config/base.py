@@ -37,9 +37,12 @@ def read_config_json(model_dir: str) -> dict:
 
 
 def architecture_name(raw: Mapping[str, Any]) -> str:
+    """The first name of ``architectures``, or the one name a file gives as ``architecture``."""
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str) and raw["architecture"]:
+        return raw["architecture"]
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json: 'architectures' must be a non-empty list of names")
+        raise ConfigError("config.json: 'architectures' must be a non-empty list of names (or 'architecture' one name)")
     return archs[0]
 
 
@@ -123,3 +126,22 @@ class Fields:
         if not isinstance(v, dict):
             raise ConfigError(f"{self.where}: '{key}' must be an object, got {v!r}")
         return Fields(v, f"{self.where}:{key}")
+
+    def mappings(self, key: str) -> list:
+        """A non-empty list of objects, each as ``Fields``."""
+        v = self._get(key, _MISSING)
+        if not isinstance(v, list) or not v or not all(isinstance(it, dict) for it in v):
+            raise ConfigError(f"{self.where}: '{key}' must be a non-empty list of objects")
+        return [Fields(it, f"{self.where}:{key}[{i}]") for i, it in enumerate(v)]
+
+    def numbers(self, key: str, count: Optional[int] = None, lo: float = -math.inf, hi: float = math.inf) -> tuple:
+        """A list of finite numbers (of ``count`` entries if given)."""
+        v = self._get(key, _MISSING)
+        if not isinstance(v, list) or any(isinstance(x, bool) or not isinstance(x, (int, float)) for x in v):
+            raise ConfigError(f"{self.where}: '{key}' must be a list of numbers, got {v!r}")
+        out = tuple(float(x) for x in v)
+        if any(math.isnan(x) or math.isinf(x) or x < lo or x > hi for x in out):
+            raise ConfigError(f"{self.where}: '{key}' holds a number out of range")
+        if count is not None and len(out) != count:
+            raise ConfigError(f"{self.where}: '{key}' has {len(out)} entries, {count} are needed")
+        return out

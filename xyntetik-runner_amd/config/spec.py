@@ -35,12 +35,13 @@ class LayerSpec:
     follow each other); ``norms`` holds the norms that arrangement has, under the names it
     gives them ("prenorm": ``mixer_norm`` and ``feed_forward_norm``; an arrangement with a
     third norm simply names three).  An arrangement may do without a mixer or without a
-    feed-forward.
+    feed-forward, and may name sequence filters (``filters``) that its sublayers' inputs pass.
     """
     mixer: Optional[PartSpec] = None
     feed_forward: Optional[PartSpec] = None
     norms: Mapping[str, PartSpec] = field(default_factory=dict)
     block: str = "prenorm"
+    filters: Mapping[str, PartSpec] = field(default_factory=dict)    # sequence filters, by the arrangement's names
 
 
 @dataclass(frozen=True)

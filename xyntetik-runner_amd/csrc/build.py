@@ -35,7 +35,8 @@ HIPCC_FLAGS = [
 UNITS: Dict[str, dict] = {
     "kernels": {
         "sources": ["errors.hip", "basic_kernels.hip", "gemm_ref.hip", "attention_ref.hip",
-                    "sampling.hip", "gemm_mfma.hip"],
+                    "sampling.hip", "gemm_mfma.hip", "sequence_kernels.hip", "recurrent_kernels.hip",
+                    "attention_pooled.hip"],
         "defines": [],
     },
 }

@@ -57,7 +57,20 @@ _PROTOS = {
     "xr_rope_table": [_p, _p, _p, _i, _i, _f, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
+    "xr_layernorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
+    "xr_causal_conv": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_polynorm": [_p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
+    "xr_rotate_rows": [_p, _p, _p, _i, _i, _i, _i, _i, _f, _p],
+    "xr_gated_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _p],
+    "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
+    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_pool_blocks": [_p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_attention_pooled": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
 }
+
+CONV_ACTIVATIONS = {None: 0, "none": 0, "silu": 1}      # XR_CONV_* of sequence_kernels.hip
+RECURRENCES = {"retention": 0, "delta": 1}              # XR_REC_* of recurrent_kernels.hip
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -573,6 +586,198 @@ class Ops:
                                                     _i, _i, _i, _i, _f, _i, _p]})
             self._attn_libs[D] = lib
         return lib
+
+    # -- row-wise and time-wise operations around the sequence mixers ----------
+    def layernorm(self, x: torch.Tensor, w: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``(x - mean) / sqrt(var + eps) * w`` of the rows of 32-bit ``x`` (or of the rows ``rows``
+        selects); ``w`` 32-bit or absent, no bias."""
+        self._dev(x, w, rows)
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+            raise KernelError("layernorm input must be float32 [rows, width] with unit column stride")
+        E = x.shape[1]
+        if w is not None and (w.dtype != torch.float32 or w.numel() != E or not w.is_contiguous()):
+            raise KernelError(f"layernorm weight must be float32 [{E}]")
+        R = x.shape[0] if rows is None else rows.numel()
+        out = torch.empty((R, E), dtype=out_dtype, device=x.device)
+        self.lib.check(self.lib.xr_layernorm(out.data_ptr(), x.data_ptr(), _ptr(w), _ptr(rows), R, E, x.stride(0),
+                                             float(eps), dtype_code(out_dtype), _stream()))
+        return out
+
+    def causal_conv(self, u: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], ctx, out_dtype: torch.dtype,
+                    residual: bool = False, activation: Optional[str] = None) -> torch.Tensor:
+        """A convolution over time on every channel of ``u [T, C]``: ``y_t = sum_j w[:, j] u_(t-taps+1+j)``
+        (plus ``u_t`` with ``residual``), then the activation.  ``state [slots + 1, taps - 1, C]`` (the
+        dtype of ``u``) holds every request's last ``taps - 1`` inputs and is brought up to date;
+        ``ctx`` gives the step's rows (``cu_q``, ``slots``, ``req_of_token``)."""
+        self._dev(u, w, state)
+        if u.dim() != 2 or u.stride(1) != 1:
+            raise KernelError("causal_conv input must be [rows, channels] with unit column stride")
+        T, Cn = u.shape
+        if w.dtype != torch.float32 or w.dim() != 2 or w.shape[0] != Cn or not w.is_contiguous():
+            raise KernelError(f"causal_conv weight must be float32 [{Cn}, taps]")
+        taps = w.shape[1]
+        if taps > 1:
+            if state is None or state.dtype != u.dtype or tuple(state.shape[1:]) != (taps - 1, Cn) or not state.is_contiguous():
+                raise KernelError(f"causal_conv state must be {u.dtype} [slots, {taps - 1}, {Cn}]")
+        if activation not in CONV_ACTIVATIONS:
+            raise KernelError(f"causal_conv: activation {activation!r} is not built (known: none, silu)")
+        out = torch.empty((T, Cn), dtype=out_dtype, device=u.device)
+        self.lib.check(self.lib.xr_causal_conv(out.data_ptr(), u.data_ptr(), w.data_ptr(), _ptr(state), ctx.cu_q.data_ptr(),
+                                               ctx.slots.data_ptr(), ctx.req_of_token.data_ptr(), T, ctx.B, Cn, taps,
+                                               u.stride(0), Cn, dtype_code(u.dtype), dtype_code(out_dtype),
+                                               1 if residual else 0, CONV_ACTIVATIONS[activation], _stream()))
+        return out
+
+    def polynorm(self, z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+        """``a N(z) + b N(z^2) + c N(z^3) + e`` per row, ``N(v) = v / sqrt(mean(v^2) + eps)``,
+        ``coef`` = (a, b, c, e) as 32-bit floats on the device."""
+        self._dev(z, coef)
+        if z.dim() != 2 or z.stride(1) != 1:
+            raise KernelError("polynorm input must be [rows, width] with unit column stride")
+        if coef.dtype != torch.float32 or coef.numel() != 4:
+            raise KernelError("polynorm takes four 32-bit coefficients")
+        T, F = z.shape
+        out = torch.empty((T, F), dtype=out_dtype, device=z.device)
+        self.lib.check(self.lib.xr_polynorm(out.data_ptr(), z.data_ptr(), coef.data_ptr(), T, F, z.stride(0), float(eps),
+                                            dtype_code(z.dtype), dtype_code(out_dtype), _stream()))
+        return out
+
+    def rotate_rows_(self, x: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], heads: int, D: int,
+                     rot: int, scale: float = 1.0) -> None:
+        """Rotate the first ``rot`` channels of every head of the 32-bit view ``x [T, heads * D]`` in
+        place (channel j pairs with j + rot/2, angle = position x ``inv_freq[j]``), then scale."""
+        self._dev(x, positions, inv_freq)
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != heads * D:
+            raise KernelError(f"rotate_rows_: x must be a float32 view [rows, {heads * D}] with unit column stride")
+        if rot and (inv_freq is None or inv_freq.numel() != rot // 2 or inv_freq.dtype != torch.float32):
+            raise KernelError(f"rotate_rows_: {rot // 2} 32-bit frequencies are needed")
+        self.lib.check(self.lib.xr_rotate_rows(x.data_ptr(), positions.data_ptr(), _ptr(inv_freq), x.shape[0], heads, D,
+                                               rot, x.stride(0), float(scale), _stream()))
+
+    def gated_rmsnorm(self, o: torch.Tensor, gate: torch.Tensor, w: Optional[torch.Tensor], H: int, Dv: int, eps: float,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+        """``o / rms(o) * w * silu(gate)`` per head: ``o [T, H * Dv]`` 32-bit and contiguous, ``gate`` a
+        32-bit view of the same shape, ``w [Dv]`` 32-bit or absent."""
+        self._dev(o, gate, w)
+        T = o.shape[0]
+        if o.dtype != torch.float32 or not o.is_contiguous() or o.shape[1] != H * Dv:
+            raise KernelError(f"gated_rmsnorm: o must be contiguous float32 [rows, {H * Dv}]")
+        if gate.dtype != torch.float32 or gate.stride(1) != 1 or tuple(gate.shape) != (T, H * Dv):
+            raise KernelError("gated_rmsnorm: the gate must be a float32 view of o's shape")
+        if w is not None and (w.dtype != torch.float32 or w.numel() != Dv):
+            raise KernelError(f"gated_rmsnorm: the weight must be float32 [{Dv}]")
+        out = torch.empty((T, H * Dv), dtype=out_dtype, device=o.device)
+        self.lib.check(self.lib.xr_gated_rmsnorm(out.data_ptr(), o.data_ptr(), gate.data_ptr(), _ptr(w), T, H, Dv,
+                                                 gate.stride(0), float(eps), dtype_code(out_dtype), _stream()))
+        return out
+
+    def delta_prepare_(self, q, k, b, a, a_log, dt_bias, G: int, H: int, D: int, q_scale: float, unit_eps: float) -> None:
+        """In place on 32-bit views (``q`` and ``k`` with one row stride, ``b`` and ``a`` with one):
+        query and key heads become unit vectors (queries times ``q_scale``), ``b`` becomes
+        ``sigmoid(b)``, ``a`` becomes ``exp(-exp(a_log) * softplus(a + dt_bias))``."""
+        self._dev(q, k, b, a, a_log, dt_bias)
+        views = (q, k, b, a)
+        if (any(v.dtype != torch.float32 or v.stride(1) != 1 for v in views) or q.stride(0) != k.stride(0)
+                or b.stride(0) != a.stride(0)):
+            raise KernelError("delta_prepare_: q and k, and b and a, must be float32 views with one row stride each")
+        if tuple(q.shape[1:]) != (G * D,) or tuple(k.shape[1:]) != (G * D,) or b.shape[1] != H or a.shape[1] != H:
+            raise KernelError("delta_prepare_: view widths do not fit the heads")
+        if a_log.dtype != torch.float32 or dt_bias.dtype != torch.float32 or a_log.numel() != H or dt_bias.numel() != H:
+            raise KernelError(f"delta_prepare_: A_log and dt_bias must be float32 [{H}]")
+        self.lib.check(self.lib.xr_delta_prepare(q.data_ptr(), k.data_ptr(), b.data_ptr(), a.data_ptr(), a_log.data_ptr(),
+                                                 dt_bias.data_ptr(), q.shape[0], G, H, D, q.stride(0), b.stride(0),
+                                                 float(q_scale), float(unit_eps), _stream()))
+
+    @staticmethod
+    def recurrence_state_shape(H: int, D: int, Dv: int):
+        """The per-request state of ``linear_recurrence``: S[4 j + r][c] of head h at ``[h, j, c, r]``."""
+        return (H, (D + 3) // 4, Dv, 4)
+
+    def linear_recurrence(self, kind: str, q, k, v, state: torch.Tensor, ctx, H: int, G: int, D: int, Dv: int,
+                          beta=None, gate=None, decay=None) -> torch.Tensor:
+        """The read-outs ``[T, H * Dv]`` (32-bit) of a linear recurrence over every request's rows,
+        from and into ``state [slots + 1, *recurrence_state_shape]``.  ``kind`` "retention":
+        ``S <- decay_h S + k v^T`` with ``decay [H]``; "delta": ``S <- g S; u = beta (v - S^T k);
+        S <- S + k u^T`` with ``beta``/``gate [T, H]``; ``o = S^T q`` after the update in both.
+        ``q, k [T, G * D]``, ``v [T, H * Dv]``: 32-bit views that share a row stride."""
+        if kind not in RECURRENCES:
+            raise KernelError(f"linear_recurrence: kind {kind!r} (known: {sorted(RECURRENCES)})")
+        self._dev(q, k, v, state, beta, gate, decay)
+        views, gates = (q, k, v), [t for t in (beta, gate) if t is not None]
+        if (any(t.dtype != torch.float32 or t.stride(1) != 1 for t in list(views) + gates)
+                or len({t.stride(0) for t in views}) != 1 or len({t.stride(0) for t in gates}) > 1):
+            raise KernelError("linear_recurrence: q, k and v, and the gates, must be float32 views with one row stride each")
+        T = q.shape[0]
+        if tuple(q.shape) != (T, G * D) or tuple(k.shape) != (T, G * D) or tuple(v.shape) != (T, H * Dv):
+            raise KernelError("linear_recurrence: view widths do not fit the heads")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != self.recurrence_state_shape(H, D, Dv) or not state.is_contiguous():
+            raise KernelError(f"linear_recurrence: state must be float32 [slots, {self.recurrence_state_shape(H, D, Dv)}]")
+        if kind == "delta":
+            if beta is None or gate is None or tuple(beta.shape) != (T, H) or tuple(gate.shape) != (T, H):
+                raise KernelError("linear_recurrence: the delta rule needs beta and gate [T, H]")
+        elif decay is None or decay.dtype != torch.float32 or decay.numel() != H:
+            raise KernelError(f"linear_recurrence: retention needs float32 decay [{H}]")
+        out = torch.empty((T, H * Dv), dtype=torch.float32, device=q.device)
+        self.lib.check(self.lib.xr_linear_recurrence(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), _ptr(beta),
+                                                     _ptr(gate), _ptr(decay), state.data_ptr(), ctx.cu_q.data_ptr(),
+                                                     ctx.slots.data_ptr(), ctx.B, H, G, D, Dv, q.stride(0),
+                                                     gates[0].stride(0) if gates else 0, RECURRENCES[kind], _stream()))
+        return out
+
+    # -- windowed attention with pooled blocks ----------------------------------
+    def qkv_store(self, q, k, v, k_cache, v_cache, ctx, group: int, H: int, Hk: int, D: int, Dv: int, page_size: int,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+        """Queries ``[T, H * D]`` in ``out_dtype``; keys ``[T, Hk * D]`` and values ``[T, Hk * Dv]`` to
+        their pages (``k``/``v`` None: this layer stores none).  Inputs are 32-bit views with one row stride."""
+        self._dev(q, k, v, k_cache, v_cache)
+        views = [t for t in (q, k, v) if t is not None]
+        if any(t.dtype != torch.float32 or t.stride(1) != 1 for t in views) or len({t.stride(0) for t in views}) != 1:
+            raise KernelError("qkv_store: q, k and v must be float32 views with one row stride")
+        T = q.shape[0]
+        writes = k is not None
+        if writes and (k_cache.dtype != out_dtype or tuple(k_cache.shape[1:]) != (Hk, page_size, D)
+                       or tuple(v_cache.shape[1:]) != (Hk, Dv, page_size)):
+            raise KernelError("qkv_store: the cache does not fit the heads")
+        table = ctx.block_table(group)
+        q_out = torch.empty((T, H * D), dtype=out_dtype, device=q.device)
+        self.lib.check(self.lib.xr_qkv_store(q_out.data_ptr(), _ptr(k_cache) if writes else None,
+                                             _ptr(v_cache) if writes else None, q.data_ptr(), _ptr(k), _ptr(v), q.stride(0),
+                                             ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), table.data_ptr(),
+                                             table.stride(0), T, H, Hk if writes else 0, D, Dv, page_size,
+                                             dtype_code(out_dtype), _stream()))
+        return q_out
+
+    def pool_blocks(self, pk, pv, k_cache, v_cache, ctx, group: int, pool_group: int, Hk: int, D: int, Dv: int, P: int,
+                    page_size: int) -> None:
+        """Write the mean key and mean value of every block of ``P`` positions that this step
+        completes into the blocks' cache (entry b of a request at place b of its table in ``pool_group``)."""
+        self._dev(pk, pv, k_cache, v_cache)
+        table, ptable = ctx.block_table(group), ctx.block_table(pool_group)
+        most = ctx.max_q_len // P + 1           # no request completes more blocks than this in one step
+        self.lib.check(self.lib.xr_pool_blocks(pk.data_ptr(), pv.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                               ctx.starts_dev.data_ptr(), ctx.cu_q.data_ptr(), table.data_ptr(),
+                                               table.stride(0), ptable.data_ptr(), ptable.stride(0), ctx.B, most, Hk, D, Dv,
+                                               P, page_size, dtype_code(k_cache.dtype), _stream()))
+
+    def attention_pooled(self, q, k_cache, v_cache, pk, pv, ctx, group: int, pool_group: Optional[int], H: int, Hk: int,
+                         D: int, Dv: int, page_size: int, scale: float, size: int, P: int) -> torch.Tensor:
+        """Attention of every token of the step over the last ``size`` keys of its request and the
+        means of the blocks of ``P`` positions that end at least ``size`` positions back (``P`` = 0: none); ``[T, H * Dv]``."""
+        self._dev(q, k_cache, v_cache, pk, pv)
+        self._contig(q, "attention queries")
+        if q.dtype != k_cache.dtype or q.dtype != v_cache.dtype:
+            raise KernelError("attention: queries and cache differ in dtype")
+        T = q.shape[0]
+        table = ctx.block_table(group)
+        ptable = ctx.block_table(pool_group) if P else None
+        out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+        self.lib.check(self.lib.xr_attention_pooled(
+            out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _ptr(pk) if P else None,
+            _ptr(pv) if P else None, ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), table.data_ptr(),
+            table.stride(0), _ptr(ptable), ptable.stride(0) if P else 0, T, H, Hk, D, Dv, page_size, float(scale),
+            int(size), int(P), dtype_code(q.dtype), _stream()))
+        return out
 
     # -- sampling ---------------------------------------------------------------
     def sample(self, logits, temp, draw, top_k=None, top_p=None, min_p=None, repeat_penalty=None,

@@ -26,7 +26,8 @@ class Model:
                 ls.block,
                 make_part("mixer", ls.mixer) if ls.mixer is not None else None,
                 make_part("feed_forward", ls.feed_forward) if ls.feed_forward is not None else None,
-                {name: make_part("norm", ps) for name, ps in ls.norms.items()}))
+                {name: make_part("norm", ps) for name, ps in ls.norms.items()},
+                {name: make_part("filter", ps) for name, ps in ls.filters.items()}))
         self.final_norm = make_part("norm", spec.final_norm)
         self.head = make_part("head", spec.head)
         self.rt: Optional[Runtime] = None
@@ -37,6 +38,8 @@ class Model:
         for ls, blk in zip(self.spec.layers, self.blocks):
             for name, ps in ls.norms.items():
                 yield ps.prefix, blk.norms[name]
+            for name, ps in ls.filters.items():
+                yield ps.prefix, blk.filters[name]
             if ls.mixer is not None:
                 yield ls.mixer.prefix, blk.mixer
             if ls.feed_forward is not None:
@@ -74,12 +77,22 @@ class Model:
 
     # ------------------------------------------------------------------ what the cache must hold
     def cache_needs(self):
-        """Per entry of the run order: (KVSpec or None, StateSpec or None, cache_of)."""
+        """Per entry of the run order: (KVSpec or None, its state, cache_of).  The state is None, the
+        mixer's one ``StateSpec``, or a mapping name -> ``StateSpec`` when the layer keeps several
+        tensors (``Block.state_specs``).  An entry that reads another entry's keys and values still
+        has state of its own."""
         kv, st, of = [], [], []
         for step in self.spec.order:
-            mixer = self.blocks[step.layer].mixer
+            block = self.blocks[step.layer]
+            mixer = block.mixer
             kv.append(mixer.kv_spec() if mixer is not None else None)
-            st.append(mixer.state_spec() if mixer is not None and step.cache_of is None else None)
+            states = block.state_specs()
+            if not states:
+                st.append(None)
+            elif list(states) == ["mixer"]:
+                st.append(states["mixer"])
+            else:
+                st.append(states)
             of.append(step.cache_of)
         return kv, st, of
 

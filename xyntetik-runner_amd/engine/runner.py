@@ -202,8 +202,7 @@ class ModelRunner:
             return
         rows = None
         for lc in self.storage.layers:
-            if lc.state is None:
-                continue
-            if rows is None:
-                rows = torch.tensor(slots, dtype=torch.int32, device=self.device)
-            self.ops.fill_rows_(lc.state, rows, len(slots), 0)
+            for state in lc.states.values():
+                if rows is None:
+                    rows = torch.tensor(slots, dtype=torch.int32, device=self.device)
+                self.ops.fill_rows_(state, rows, len(slots), 0)

@@ -22,6 +22,8 @@ Families and what each must offer:
   residual stream (the default calls ``forward``; a part with a fused epilogue
   overrides it).
 * ``FeedForward``: ``forward(ctx, h) -> y`` and ``forward_add(ctx, h, residual)``.
+* ``SequenceFilter``: ``forward(ctx, state, h) -> h'``: what a sublayer reads passes through it on
+  its way from the norm; ``state_spec()`` says what it carries from token to token.
 * ``Block``: the arrangement; it names its norms (``norm_names``), may do without a mixer or a
   feed-forward, and ``forward(ctx, cache, x)`` updates ``x`` in place.
 
@@ -67,18 +69,36 @@ class KVSpec:
 
     Layers whose specs are equal share a group: one pool of pages and one block
     table per request.  ``window`` = None keeps every key; a number keeps only
-    the pages that the last ``window`` positions touch.
+    the pages that the last ``window`` positions touch.  ``v_head_dim``: the size of a
+    value where it differs from a key's.  ``pooled`` = P: beside its keys and values the
+    layer keeps one mean key and one mean value for every block of P positions, in a
+    cache of their own whose group has ``stride`` P (one entry for every ``stride``
+    positions a request has filled, never given back while the request lives).
     """
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+    pooled: Optional[int] = None
+    stride: int = 1
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_head_dim if self.v_head_dim is not None else self.head_dim
+
+    def pooled_spec(self) -> Optional["KVSpec"]:
+        """The group that holds this spec's block means."""
+        if not self.pooled:
+            return None
+        return KVSpec(self.num_kv_heads, self.head_dim, None, self.v_head_dim, None, int(self.pooled))
 
 
 @dataclass(frozen=True)
 class StateSpec:
-    """Fixed-size state per request (one slot per live request)."""
+    """Fixed-size state per request (one slot per live request).  ``dtype`` None: the engine's
+    compute dtype."""
     shape: Tuple[int, ...]
-    dtype: torch.dtype = torch.float32
+    dtype: Optional[torch.dtype] = torch.float32
 
 
 class Part:
@@ -148,7 +168,9 @@ class Mixer(Part):
         owning row ``ctx.slots[b]`` (on the device; zero when the request first uses it).  A mixer
         that finds its rows through ``ctx.slots`` can be recorded into a HIP graph, where the rows
         that pad a batch use the last state row, which is nobody's; one that reads the slots on
-        the host (``ctx.slots_host``, absent in a recorded step) sets ``capturable = False``."""
+        the host (``ctx.slots_host``, absent in a recorded step) sets ``capturable = False``.
+        A mixer with several tensors of state returns a mapping name -> ``StateSpec`` and finds them
+        in ``cache.states`` under ``"mixer." + name``."""
         return None
 
     def forward(self, ctx, cache, h: torch.Tensor) -> torch.Tensor:
@@ -164,6 +186,18 @@ class Mixer(Part):
         """``forward_add``, then ``norm`` of the updated residual stream."""
         self.forward_add(ctx, cache, h, residual)
         return norm.forward(ctx, residual)
+
+
+class SequenceFilter(Part):
+    """What a sublayer's input passes through on its way from the norm, with the inputs it carries
+    from token to token as state (a short convolution over time, say).  A block arrangement names
+    its filters as it names its norms; ``forward(ctx, state, h) -> h'`` in the compute dtype."""
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, ctx, state: Optional[torch.Tensor], h: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
 
 
 class FeedForward(Part):
@@ -188,26 +222,52 @@ class Block:
 
     #: the norms this arrangement has, by the names a ``LayerSpec`` gives them
     norm_names: Tuple[str, ...] = ()
+    #: the sequence filters it has, likewise
+    filter_names: Tuple[str, ...] = ()
     needs_mixer = True
-    needs_feed_forward = True
+    #: True, False, or None for an arrangement that runs with or without a feed-forward
+    needs_feed_forward: Optional[bool] = True
 
-    def __init__(self, mixer: Optional[Mixer], feed_forward: Optional[FeedForward], norms: Dict[str, Norm]):
+    def __init__(self, mixer: Optional[Mixer], feed_forward: Optional[FeedForward], norms: Dict[str, Norm],
+                 filters: Optional[Dict[str, "SequenceFilter"]] = None):
         kind = type(self).__name__
-        if (mixer is None) == self.needs_mixer or (feed_forward is None) == self.needs_feed_forward:
+        if (mixer is None) == self.needs_mixer or (self.needs_feed_forward is not None
+                                                   and (feed_forward is None) == self.needs_feed_forward):
             raise ValueError(f"{kind}: this arrangement has {'a' if self.needs_mixer else 'no'} mixer and "
                              f"{'a' if self.needs_feed_forward else 'no'} feed-forward")
         if set(norms) != set(self.norm_names):
             raise ValueError(f"{kind}: this arrangement has the norms {sorted(self.norm_names)}, "
                              f"the layer names {sorted(norms)}")
-        self.mixer, self.feed_forward, self.norms = mixer, feed_forward, dict(norms)
+        filters = dict(filters or {})
+        if set(filters) != set(self.filter_names):
+            raise ValueError(f"{kind}: this arrangement has the filters {sorted(self.filter_names)}, "
+                             f"the layer names {sorted(filters)}")
+        self.mixer, self.feed_forward, self.norms, self.filters = mixer, feed_forward, dict(norms), filters
 
     def parts(self):
         """Every part of the layer by name."""
         out = dict(self.norms)
+        out.update(self.filters)
         if self.mixer is not None:
             out["mixer"] = self.mixer
         if self.feed_forward is not None:
             out["feed_forward"] = self.feed_forward
+        return out
+
+    def state_specs(self) -> Dict[str, StateSpec]:
+        """Every tensor of per-request state the layer keeps, by the name it is found under in
+        ``cache.states``: the mixer's as "mixer" (or "mixer.<name>" if it has several), a filter's
+        under the filter's name."""
+        out: Dict[str, StateSpec] = {}
+        st = self.mixer.state_spec() if self.mixer is not None else None
+        if isinstance(st, StateSpec):
+            out["mixer"] = st
+        elif st:
+            out.update({"mixer." + k: v for k, v in st.items()})
+        for name, f in self.filters.items():
+            fs = f.state_spec()
+            if fs is not None:
+                out[name] = fs
         return out
 
     #: True if ``forward`` also takes ``h`` (the result of this block's first norm, made by the
@@ -240,7 +300,7 @@ class Runtime:
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
     "norm": {}, "position": {}, "qk_transform": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {},
-    "head": {},
+    "head": {}, "filter": {},
 }
 
 
@@ -265,6 +325,10 @@ def register_qk_transform(kind, factory, replace=False):
 
 def register_mixer(kind, factory, replace=False):
     _register("mixer", kind, factory, replace)
+
+
+def register_filter(kind, factory, replace=False):
+    _register("filter", kind, factory, replace)
 
 
 def register_feed_forward(kind, factory, replace=False):
@@ -295,9 +359,12 @@ def make_part(family: str, spec) -> Any:
     return reg[spec.kind](**spec.params)
 
 
-def make_block(kind: str, mixer, feed_forward, norms) -> Block:
-    """The arrangement ``kind`` around the given parts (``norms``: name -> norm)."""
+def make_block(kind: str, mixer, feed_forward, norms, filters=None) -> Block:
+    """The arrangement ``kind`` around the given parts (``norms``: name -> norm; ``filters``: name ->
+    sequence filter, for an arrangement that has any)."""
     reg = _REGISTRIES["block"]
     if kind not in reg:
         raise ValueError(f"no block arrangement {kind!r}; registered: {sorted(reg)}")
+    if filters:
+        return reg[kind](mixer, feed_forward, norms, filters)
     return reg[kind](mixer, feed_forward, norms)

@@ -3,6 +3,10 @@
 "prenorm": ``x += mixer(norm(x)); x += feed_forward(norm(x))`` — norm, projections,
 rotation, cache write, attention, output, add, norm, feed-forward, add, every layer
 alike (src/model.c:6168-6473).
+
+"prenorm_filtered": the same, but what each sublayer reads goes through a sequence filter first:
+``x += mixer(filter_m(norm(x))); x += feed_forward(filter_f(norm(x)))``.  A layer of it may come
+without a feed-forward.
 """
 from __future__ import annotations
 
@@ -48,4 +52,27 @@ class PreNormBlock(Block):
         return add_norm(ctx, h, x, next_norm, defer=defer)
 
 
+class FilteredPreNormBlock(Block):
+    norm_names = ("mixer_norm", "feed_forward_norm")
+    filter_names = ("mixer_filter", "feed_forward_filter")
+    needs_feed_forward = None       # with or without; the second norm and filter then do nothing
+
+    def forward(self, ctx, cache, x):
+        h = self.norms["mixer_norm"].forward(ctx, x)
+        h = self.filters["mixer_filter"].forward(ctx, cache.states.get("mixer_filter"), h)
+        self.mixer.forward_add(ctx, cache, h, x)
+        if self.feed_forward is None:
+            return
+        h = self.norms["feed_forward_norm"].forward(ctx, x)
+        h = self.filters["feed_forward_filter"].forward(ctx, cache.states.get("feed_forward_filter"), h)
+        self.feed_forward.forward_add(ctx, h, x)
+
+    def state_specs(self):
+        out = super().state_specs()
+        if self.feed_forward is None:
+            out.pop("feed_forward_filter", None)
+        return out
+
+
 register_block("prenorm", PreNormBlock)
+register_block("prenorm_filtered", FilteredPreNormBlock)

@@ -4,6 +4,10 @@
 ``gate`` and ``up`` are kept as one ``[2F, E]`` matrix so that one product makes both;
 the reference does the reverse for a checkpoint that stores them fused
 (``slice_rows``, src/model.c:238-248).
+
+Dense feed-forward: ``down(act(up(h)))`` with an activation over the whole row.  "polynorm":
+``a N(z) + b N(z^2) + c N(z^3) + e`` with four learned numbers, powers element by element and
+``N(v) = v / sqrt(mean(v^2) + eps)`` over the row, in 32-bit.
 """
 from __future__ import annotations
 
@@ -68,4 +72,41 @@ class GatedMLP(FeedForward):
                                               self.rt.dtype, bias=self.b_down, defer=defer)
 
 
+class DenseMLP(FeedForward):
+    ACTIVATIONS = ("polynorm",)
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "polynorm", eps: float = 1e-5,
+                 up_name: str = "up", down_name: str = "down", act_name: str = "act"):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"dense feed-forward: activation {activation!r} is not built (known: {list(self.ACTIVATIONS)})")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation, self.eps = activation, float(eps)
+        self.names = (up_name, down_name, act_name)
+        self.w_up = self.w_down = self.coef = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E, F = self.hidden_size, self.intermediate_size
+        u, d, a = self.names
+        return {u: ParamSpec((F, E)), d: ParamSpec((E, F)), a: ParamSpec((4,), role="vector", init="ones_jitter")}
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        u, d, a = self.names
+        self.w_up = rt.ops.pack_weight(tensors[u])
+        self.w_down = rt.ops.pack_weight(tensors[d])
+        self.coef = tensors[a].float().contiguous()
+
+    def _hidden(self, ctx, h):
+        # the row's statistics are of the unrounded products
+        z = self.rt.ops.linear(h, self.w_up, out_dtype=torch.float32)
+        return self.rt.ops.polynorm(z, self.coef, self.eps, self.rt.dtype)
+
+    def forward(self, ctx, h):
+        return self.rt.ops.linear(self._hidden(ctx, h), self.w_down)
+
+    def forward_add(self, ctx, h, residual) -> None:
+        self.rt.ops.linear(self._hidden(ctx, h), self.w_down, out=residual, accumulate=True)
+
+
 register_feed_forward("gated_mlp", GatedMLP)
+register_feed_forward("dense_mlp", DenseMLP)

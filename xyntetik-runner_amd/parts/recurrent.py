@@ -1,0 +1,167 @@
+"""Mixers whose memory is a matrix of state per request and head, carried from token to token
+in 32-bit floats (``Ops.linear_recurrence``), read out as ``o = S^T q`` after the token's update.
+
+``Retention``: linear attention with one fixed decay a head and neither softmax nor denominator.
+``q = Wq h``, ``k = Wk h`` (H heads of D), ``v = Wv h`` (H heads of Dv); an optional rotation of the
+first channels of q and k; k times ``D^-1/2`` after it; ``S <- decay_h S + k v^T``.  Every head's
+read-out is divided by its root mean square, then times ``silu(Wg h)``, then ``Wo``.
+
+``GatedDelta``: the gated delta rule.  ``q``, ``k`` (G heads of D; head h reads head ``h // (H / G)``)
+and ``v`` (H heads of Dv) each pass a short causal convolution over time and SiLU; q and k become
+unit vectors ``x / sqrt(sum(x^2) + 1e-6)``, q also times ``D^-1/2``; ``beta = sigmoid(Wb h)`` and
+``g = exp(-exp(A_log_h) * softplus(Wa h + dt_bias_h))`` a head; ``S <- g S; u = beta (v - S^T k);
+S <- S + k u^T``.  The read-out is divided by its root mean square, times a weight over Dv that
+the heads share, times ``silu(Wg h)``, then ``Wo``.
+
+Both keep their projections in 32 bits from the product to the recurrence: what enters a
+recurrence is not rounded on the way.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Sequence
+
+import torch
+
+from .base import Mixer, ParamSpec, StateSpec, make_part, register_mixer
+
+MAX_KEY_DIM = 256       # a column of the state is kept in the registers of four lanes
+
+
+def _check_sizes(what: str, heads: int, kv_heads: int, dim: int, vdim: int) -> None:
+    if heads < 1 or kv_heads < 1 or heads % kv_heads:
+        raise ValueError(f"{what}: {heads} heads are not a multiple of {kv_heads} key heads")
+    if not (1 <= dim <= MAX_KEY_DIM) or vdim < 1:
+        raise ValueError(f"{what}: key size {dim} (1 to {MAX_KEY_DIM}), value size {vdim}")
+
+
+class Retention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, decay: Sequence[float],
+                 eps: float, position=None, q_name: str = "q", k_name: str = "k", v_name: str = "v",
+                 g_name: str = "g", o_name: str = "o"):
+        _check_sizes("retention", num_heads, num_heads, head_dim, v_head_dim)
+        if len(decay) != num_heads:
+            raise ValueError(f"retention: {len(decay)} decays for {num_heads} heads")
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.head_dim, self.v_head_dim = int(head_dim), int(v_head_dim)
+        self.decay_values, self.eps = [float(d) for d in decay], float(eps)
+        self.position = make_part("position", position) if position is not None else None
+        self.names = (q_name, k_name, v_name, g_name, o_name)
+        self.qk_size, self.v_size = self.num_heads * self.head_dim, self.num_heads * self.v_head_dim
+
+    @property
+    def capturable(self) -> bool:
+        return self.position is None or self.position.capturable
+
+    def state_spec(self):
+        from ..csrc.ops import Ops
+        return StateSpec(Ops.recurrence_state_shape(self.num_heads, self.head_dim, self.v_head_dim), torch.float32)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E = self.hidden_size
+        q, k, v, g, o = self.names
+        return {q: ParamSpec((self.qk_size, E)), k: ParamSpec((self.qk_size, E)), v: ParamSpec((self.v_size, E)),
+                g: ParamSpec((self.v_size, E)), o: ParamSpec((E, self.v_size))}
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        q, k, v, g, o = self.names
+        self.w_in = rt.ops.pack_weight(torch.cat([tensors[q], tensors[k], tensors[v], tensors[g]], dim=0).contiguous())
+        self.w_out = rt.ops.pack_weight(tensors[o])
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=rt.device)
+        if self.position is not None:
+            self.position.bind({}, rt)
+            rot = self.position.rotary()
+            if rot is None or rot.interleaved or rot.mscale != 1.0:
+                raise ValueError("retention rotates channel j with j + dims/2 by a plain frequency table")
+
+    def _read_out(self, ctx, cache, h):
+        ops = self.rt.ops
+        H, D, Dv, QK, V = self.num_heads, self.head_dim, self.v_head_dim, self.qk_size, self.v_size
+        proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
+        q, k, v, gate = proj[:, :QK], proj[:, QK:2 * QK], proj[:, 2 * QK:2 * QK + V], proj[:, 2 * QK + V:]
+        rot = self.position.rotary() if self.position is not None else None
+        if rot is not None:
+            ops.rotate_rows_(q, ctx.positions, rot.inv_freq, H, D, rot.rotary_dim, 1.0)
+        ops.rotate_rows_(k, ctx.positions, rot.inv_freq if rot else None, H, D, rot.rotary_dim if rot else 0, D ** -0.5)
+        o = ops.linear_recurrence("retention", q, k, v, cache.state, ctx, H, H, D, Dv, decay=self.decay)
+        return ops.gated_rmsnorm(o, gate, None, H, Dv, self.eps, self.rt.dtype)
+
+    def forward(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out)
+
+    def forward_add(self, ctx, cache, h, residual) -> None:
+        self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
+
+
+class GatedDelta(Mixer):
+    UNIT_EPS = 1e-6
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
+                 conv_taps: int, eps: float, q_name: str = "q", k_name: str = "k", v_name: str = "v", b_name: str = "b",
+                 a_name: str = "a", a_log_name: str = "A_log", dt_bias_name: str = "dt_bias", norm_name: str = "norm",
+                 g_name: str = "g", o_name: str = "o", conv_suffix: str = ".conv"):
+        _check_sizes("gated delta rule", num_heads, num_kv_heads, head_dim, v_head_dim)
+        if not (1 <= int(conv_taps) <= 16):
+            raise ValueError(f"gated delta rule: {conv_taps} convolution taps (1 to 16)")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.v_head_dim = int(head_dim), int(v_head_dim)
+        self.conv_taps, self.eps = int(conv_taps), float(eps)
+        self.names = dict(q=q_name, k=k_name, v=v_name, b=b_name, a=a_name, a_log=a_log_name, dt_bias=dt_bias_name,
+                          norm=norm_name, g=g_name, o=o_name)
+        self.conv_suffix = conv_suffix
+        self.qk_size, self.v_size = self.num_kv_heads * self.head_dim, self.num_heads * self.v_head_dim
+        self.conv_size = 2 * self.qk_size + self.v_size
+
+    def state_spec(self):
+        from ..csrc.ops import Ops
+        out = {"S": StateSpec(Ops.recurrence_state_shape(self.num_heads, self.head_dim, self.v_head_dim), torch.float32)}
+        if self.conv_taps > 1:
+            out["conv"] = StateSpec((self.conv_taps - 1, self.conv_size), torch.float32)
+        return out
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E, H, n = self.hidden_size, self.num_heads, self.names
+        specs = {}
+        for key, rows in (("q", self.qk_size), ("k", self.qk_size), ("v", self.v_size)):
+            specs[n[key]] = ParamSpec((rows, E))
+            specs[n[key] + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal")
+        specs[n["b"]] = ParamSpec((H, E))
+        specs[n["a"]] = ParamSpec((H, E))
+        specs[n["a_log"]] = ParamSpec((H,), role="vector", init="zeros")
+        specs[n["dt_bias"]] = ParamSpec((H,), role="vector", init="zeros")
+        specs[n["norm"]] = ParamSpec((self.v_head_dim,), role="vector", init="ones_jitter")
+        specs[n["g"]] = ParamSpec((self.v_size, E))
+        specs[n["o"]] = ParamSpec((E, self.v_size))
+        return specs
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        n = self.names
+        self.w_in = rt.ops.pack_weight(torch.cat([tensors[n[key]] for key in ("q", "k", "v", "g", "b", "a")], dim=0).contiguous())
+        self.w_conv = torch.cat([tensors[n[key] + self.conv_suffix].float() for key in ("q", "k", "v")], dim=0).contiguous()
+        self.a_log = tensors[n["a_log"]].float().contiguous()
+        self.dt_bias = tensors[n["dt_bias"]].float().contiguous()
+        self.w_norm = tensors[n["norm"]].float().contiguous()
+        self.w_out = rt.ops.pack_weight(tensors[n["o"]])
+
+    def _read_out(self, ctx, cache, h):
+        ops = self.rt.ops
+        H, G, D, Dv, QK, V, C = (self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim, self.qk_size,
+                                 self.v_size, self.conv_size)
+        proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
+        y = ops.causal_conv(proj[:, :C], self.w_conv, cache.states.get("mixer.conv"), ctx, torch.float32, activation="silu")
+        q, k, v = y[:, :QK], y[:, QK:2 * QK], y[:, 2 * QK:]
+        gate, b, a = proj[:, C:C + V], proj[:, C + V:C + V + H], proj[:, C + V + H:]
+        ops.delta_prepare_(q, k, b, a, self.a_log, self.dt_bias, G, H, D, D ** -0.5, self.UNIT_EPS)
+        o = ops.linear_recurrence("delta", q, k, v, cache.states["mixer.S"], ctx, H, G, D, Dv, beta=b, gate=a)
+        return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype)
+
+    def forward(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out)
+
+    def forward_add(self, ctx, cache, h, residual) -> None:
+        self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
+
+
+register_mixer("retention", Retention)
+register_mixer("gated_delta", GatedDelta)

@@ -63,7 +63,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to the page size)")
     ap.add_argument("--page-size", type=int, default=64, help="positions per cache page (a power of two, default 64)")
-    ap.add_argument("--max-requests", type=int, default=16, help="most requests live at a time")
+    ap.add_argument("--max-requests", type=int, default=4, help="most requests live at a time (state slots)")
     args = ap.parse_args(argv)
     from .engine.runner import ModelRunner
     runner = ModelRunner.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens,
