@@ -1,0 +1,177 @@
+"""Suripel models through the engine against the plain implementation (``plain_suripel``):
+whole prompts, prompts with their last tokens one by one, portions down to two tokens, mixed
+batches in pools so small that pages and state slots are used again, long decoding through
+recorded steps, and greedy generation through the engine's own entry point and scheduler.
+Three configurations that differ in every size and constant (``suripel_tiny``)."""
+import io
+
+import numpy as np
+import pytest
+import torch
+
+import plain_suripel as S
+import traces
+from suripel_tiny import CONFIGS, make_model
+from tiny import logit_error, prompt_ids
+
+pytestmark = pytest.mark.gpu
+
+# fraction of the mean logit range: (max, mean)
+TOL = {"float32": (2e-5, 2e-6), "bfloat16": (3e-2, 4e-3)}
+# prompt lengths (the rest of every request is given "decoded" tokens) and how many of those
+WORKLOAD = {
+    "S1": ([1, 4, 23, 64, 150], 20),        # 1 and 4: shorter than the taps; 64: ends on a page of 64, 16 and 8
+    "S2": ([2, 9, 31, 100], 26),
+    "S3": ([3, 70, 129, 330], 40),          # past several blocks, windows and pages of 64
+}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for which in WORKLOAD:
+        d = make_model(which, str(tmp_path_factory.mktemp("suripel" + which)))
+        cfg, w = S.load_folder(d)
+        lens, extra = WORKLOAD[which]
+        reqs = {f"r{i}": prompt_ids(n + extra, cfg["vocab"], 300 + i) for i, n in enumerate(lens)}
+        plens = {f"r{i}": n for i, n in enumerate(lens)}
+        want = {rid: S.forward(cfg, w, toks) for rid, toks in reqs.items()}
+        out[which] = (d, cfg, w, reqs, plens, want)
+    return out
+
+
+def poison(runner):
+    """Old keys, old means and old state must never show: everything starts as NaN."""
+    for lc in runner.storage.layers:
+        for st in lc.states.values():
+            st.fill_(float("nan"))
+        if lc.owns and lc.k is not None:
+            lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
+        if lc.pool_owns:
+            lc.pool_k.fill_(float("nan")); lc.pool_v.fill_(float("nan"))
+
+
+def run_replay(model_dir, dtype, steps, tmp_path, page_size, max_requests=4, max_tokens=None, use_graphs=True):
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    from xyntetik_runner_amd.trace import replay
+    mt = max_tokens or traces.max_live_tokens(steps, max(64, page_size))
+    runner = ModelRunner.from_folder(model_dir, dtype=dtype, max_tokens=mt, page_size=page_size, max_requests=max_requests,
+                                     use_graphs=use_graphs)
+    poison(runner)
+    out = str(tmp_path / "out")
+    replay(runner, traces.to_lines(steps), out, report=io.StringIO())
+    runner.manager.check()
+    assert not runner.manager.requests and runner.manager.all_free()
+    return out, runner
+
+
+def check(got, want, dtype, what):
+    assert set(got) == set(want)
+    for rid in want:
+        assert np.isfinite(got[rid]).all(), f"{what} {rid}: a logit is not finite"
+        mx, mean = logit_error(got[rid], want[rid])
+        assert mx <= TOL[dtype][0] and mean <= TOL[dtype][1], f"{what} {rid} ({dtype}): max {mx:.3g} mean {mean:.3g}"
+
+
+SCHEDULES = ["whole", "tail", "portions", "mixed"]
+
+
+def steps_for(schedule, reqs, plens, extra):
+    if schedule == "whole":
+        return traces.whole(reqs)
+    if schedule == "tail":
+        return traces.tail_one_by_one(reqs, tail=extra)
+    if schedule == "portions":
+        return traces.portions(reqs)
+    return traces.mixed(reqs, plens, max_live=3, seed=5)
+
+
+@pytest.mark.parametrize("schedule", SCHEDULES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which,page_size", [("S1", 16), ("S2", 8), ("S3", 64)])
+def test_every_way_of_cutting_gives_the_plain_logits(models, tmp_path, which, page_size, dtype, schedule):
+    d, cfg, w, reqs, plens, want = models[which]
+    steps = steps_for(schedule, reqs, plens, WORKLOAD[which][1])
+    out, runner = run_replay(d, dtype, steps, tmp_path, page_size, max_requests=3)
+    check(traces.collect(steps, out, cfg["vocab"]), want, dtype, f"{which} {schedule}")
+    if schedule == "tail":
+        assert runner.graphs.replays > 0, "single tokens went through no recorded step"
+
+
+def test_mixed_batch_equals_each_request_alone_bit_for_bit_in_kind(models, tmp_path):
+    """What a request's logits are does not depend on its neighbours in the batch beyond rounding:
+    the mixed schedule against the same requests alone, engine against engine, in 32-bit."""
+    d, cfg, w, reqs, plens, want = models["S3"]
+    alone, _ = run_replay(d, "float32", traces.portions(reqs), tmp_path / "a", 64)
+    steps = traces.mixed(reqs, plens, max_live=4, seed=9)
+    mixed, _ = run_replay(d, "float32", steps, tmp_path / "m", 64)
+    a = traces.collect(traces.portions(reqs), alone, cfg["vocab"])
+    m = traces.collect(steps, mixed, cfg["vocab"])
+    for rid in reqs:
+        mx, _ = logit_error(m[rid], a[rid])
+        assert mx <= 5e-6, f"{rid}: {mx:.3g}"
+
+
+def test_slots_and_pages_are_used_again(models, tmp_path):
+    """Two state slots and pools for the two longest requests: every request after the first two
+    runs in a slot and in pages that another has used, which were filled with its state and keys."""
+    d, cfg, w, reqs, plens, want = models["S1"]
+    steps = traces.mixed(reqs, plens, max_live=2, seed=3)
+    out, runner = run_replay(d, "float32", steps, tmp_path, 8, max_requests=2)
+    assert runner.manager.slots.size == 2
+    check(traces.collect(steps, out, cfg["vocab"]), want, "float32", "reuse")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_through_recorded_steps(models, tmp_path, dtype):
+    """A short prompt and 300 tokens one by one: the windows, several blocks and pages of every
+    attention layer pass over decoded tokens, and the recurrent state is carried 300 times."""
+    d, cfg, w, reqs, plens, want = models["S3"]
+    toks = prompt_ids(310, cfg["vocab"], 77)
+    wanted = S.forward(cfg, w, toks)
+    steps = traces.tail_one_by_one({"long": toks}, tail=300)
+    out, runner = run_replay(d, dtype, steps, tmp_path, 16)
+    assert runner.graphs.replays >= 290
+    check(traces.collect(steps, out, cfg["vocab"]), {"long": wanted}, dtype, "long decoding")
+
+
+def test_eager_and_recorded_steps_agree(models, tmp_path):
+    d, cfg, w, reqs, plens, want = models["S2"]
+    steps = traces.tail_one_by_one(reqs, tail=26)
+    a, _ = run_replay(d, "float32", steps, tmp_path / "g", 8, use_graphs=True)
+    b, _ = run_replay(d, "float32", steps, tmp_path / "e", 8, use_graphs=False)
+    ga, gb = traces.collect(steps, a, cfg["vocab"]), traces.collect(steps, b, cfg["vocab"])
+    for rid in reqs:
+        assert np.array_equal(ga[rid], gb[rid]), rid
+
+
+@pytest.mark.parametrize("which", ["S1", "S3"])
+def test_greedy_generation_through_the_entry_point(models, which):
+    """``LLM.generate``: scheduler, portions under a token budget, sampling on the device."""
+    from xyntetik_runner_amd import LLM, SamplingParams
+    d, cfg, w, reqs, plens, want = models[which]
+    prompts = [prompt_ids(n, cfg["vocab"], 500 + n) for n in (3, 21, 40)]
+    wanted = [S.greedy(cfg, w, p, 8) for p in prompts]
+    llm = LLM(d, dtype="float32", max_tokens=512, page_size=16, max_batched_tokens=16, max_running=2)
+    got = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=8))
+    assert got == wanted
+    assert llm.runner.manager.all_free()
+
+
+def test_model_is_built_from_its_config(models):
+    from xyntetik_runner_amd.config import load_config
+    from xyntetik_runner_amd.engine.model import Model
+    d, cfg, w, *_ = models["S1"]
+    arch, c = load_config(d)
+    assert arch.name == "Suripel"
+    spec = arch.build_spec(c)
+    exp = Model.expected_tensors(spec)
+    assert sorted(exp) == sorted(w)                                 # (the random-weights mode writes optional tensors too)
+    assert sorted(n for n, ps in exp.items() if ps.optional) == ["l2.canon2", "l2.norm2"]
+    assert "l3.mix.k" not in exp and "l3.mix.q.conv" in exp         # a reader has queries only
+    assert "l2.mlp.up" not in exp                                   # a layer without a feed-forward
+    kv, st, of = Model(spec).cache_needs()
+    assert of == [None, None, None, 1, None]
+    assert kv[1].window == 9 and kv[1].pooled == 5 and kv[3].pooled == 7 and kv[1].v_head_dim == 24
+    assert set(st[0]) == {"mixer.S", "mixer.conv", "mixer_filter", "feed_forward_filter"}
+    assert set(st[2]) == {"mixer", "mixer_filter"}                  # no feed-forward: no second filter's state

@@ -54,8 +54,8 @@ class ParamSpec:
     ``role``: "matrix" tensors are kept in the engine's compute dtype; "vector"
     tensors keep 32 bits if the file stores them so (bfloat16 otherwise, in a
     bfloat16 engine); "int" tensors become int32.
-    ``init`` tells the random-weights mode what to write: "normal", "ones",
-    "ones_jitter" (1 + N(0, jitter)) or "zeros".
+    ``init`` tells the random-weights mode what to write: "normal" (the model's deviation),
+    "normal:<s>" (deviation s), "ones", "ones_jitter" (1 + N(0, jitter)) or "zeros".
     """
     shape: Tuple[int, ...]
     role: str = "matrix"

@@ -29,7 +29,7 @@ class CausalConv(SequenceFilter):
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {self.weight_name: ParamSpec((self.channels, self.taps), role="vector", init="normal", optional=self.optional)}
+        return {self.weight_name: ParamSpec((self.channels, self.taps), role="vector", init="normal:0.4", optional=self.optional)}
 
     def state_spec(self) -> Optional[StateSpec]:
         if self.taps <= 1:

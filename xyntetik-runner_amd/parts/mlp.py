@@ -87,7 +87,7 @@ class DenseMLP(FeedForward):
     def param_specs(self) -> Dict[str, ParamSpec]:
         E, F = self.hidden_size, self.intermediate_size
         u, d, a = self.names
-        return {u: ParamSpec((F, E)), d: ParamSpec((E, F)), a: ParamSpec((4,), role="vector", init="ones_jitter")}
+        return {u: ParamSpec((F, E)), d: ParamSpec((E, F)), a: ParamSpec((4,), role="vector", init="normal:0.5")}
 
     def bind(self, tensors, rt) -> None:
         self.rt = rt

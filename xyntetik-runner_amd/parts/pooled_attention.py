@@ -79,7 +79,7 @@ class PooledWindowAttention(Mixer):
         specs = {}
         for name, rows in self._projections():
             specs[name] = ParamSpec((rows, E))
-            specs[name + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal")
+            specs[name + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal:0.6")
         specs[self.names[3]] = ParamSpec((E, self.num_heads * self.v_head_dim))
         return specs
 

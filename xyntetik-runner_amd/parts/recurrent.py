@@ -124,11 +124,11 @@ class GatedDelta(Mixer):
         specs = {}
         for key, rows in (("q", self.qk_size), ("k", self.qk_size), ("v", self.v_size)):
             specs[n[key]] = ParamSpec((rows, E))
-            specs[n[key] + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal")
+            specs[n[key] + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal:0.6")
         specs[n["b"]] = ParamSpec((H, E))
         specs[n["a"]] = ParamSpec((H, E))
-        specs[n["a_log"]] = ParamSpec((H,), role="vector", init="zeros")
-        specs[n["dt_bias"]] = ParamSpec((H,), role="vector", init="zeros")
+        specs[n["a_log"]] = ParamSpec((H,), role="vector", init="normal:0.5")
+        specs[n["dt_bias"]] = ParamSpec((H,), role="vector", init="normal:0.5")
         specs[n["norm"]] = ParamSpec((self.v_head_dim,), role="vector", init="ones_jitter")
         specs[n["g"]] = ParamSpec((self.v_size, E))
         specs[n["o"]] = ParamSpec((E, self.v_size))

@@ -36,6 +36,8 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, std: float, jitter: flo
     dt = torch.int32 if spec.role == "int" else (vector_dtype if spec.role == "vector" else matrix_dtype)
     if spec.init == "normal":
         t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=dev) * std
+    elif spec.init.startswith("normal:"):       # a deviation of the tensor's own, whatever the model's
+        t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=dev) * float(spec.init[7:])
     elif spec.init == "ones":
         t = torch.ones(spec.shape, dtype=torch.float32, device=dev)
     elif spec.init == "ones_jitter":
