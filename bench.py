@@ -283,6 +283,105 @@ def measure_prefill_in_portions(runner, cfg, T, portion, seed):
     return best
 
 
+def suripel_config(width, layers, vocab=32000):
+    """A Suripel model of real layer sizes: heads of 128, four query heads a key/value head, a
+    window of 1,024 with blocks of 64, every mixer in turn (the second attention of each six reads
+    the first one's keys and values), a dense feed-forward with as many weights as a gated one of
+    3.5 x width."""
+    H = width // 128
+    ff = {"kind": "dense", "ff": int(width * 5.25)}
+
+    def attn(kv_from=None):
+        m = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "conv": 4, "scale": 128 ** -0.5,
+             "mask": {"size": 1024, "pool": 64}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "attention", "mixer": m, "mlp": ff}
+    delta = {"type": "delta", "mixer": {"heads": H, "kv_heads": max(1, H // 2), "dim": 128, "vdim": 128, "conv": 4}, "mlp": ff}
+    ret = {"type": "retention", "mixer": {"heads": H, "dim": 128, "vdim": 128, "decay": [1 - 2.0 ** (-5 - 5 * i / H) for i in range(H)],
+                                          "rot": {"dims": 128, "base": 1e6}}, "mlp": ff}
+    out = []
+    for i in range(layers):
+        k = i % 6
+        out.append(attn() if k == 0 else attn(kv_from=i - 4) if k == 4 else delta if k in (1, 5) else ret)
+    return {"architecture": "Suripel", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "layers": out}
+
+
+def llama_like(width, layers, vocab=32000):
+    """The closest existing model at equal size: the Llama decoder with the same width, layers, heads and weights a layer."""
+    return dict(LLAMA_3_1_8B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=width // 128,
+                num_key_value_heads=max(1, width // 512), head_dim=128, intermediate_size=int(width * 3.5), vocab_size=vocab,
+                rope_scaling=None, max_position_embeddings=8192)
+
+
+def measure_design(runner, vocab, prompt_len, batches, steps, seed):
+    """(seconds for a prompt of ``prompt_len`` tokens in one step, {batch: seconds a decode step}) through the
+    step function: the median of five prompts, and ``steps`` steps of single tokens (recorded graphs) behind
+    ``prompt_len`` cached tokens a request."""
+    import numpy as np
+    import torch
+    from xyntetik_runner_amd.engine.batch import StepEntry
+    rng = np.random.default_rng(seed)
+    toks = lambda n: [int(t) for t in rng.integers(0, vocab, size=n)]
+    times = []
+    for r in range(6):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = runner.step([StepEntry(("p", r), toks(prompt_len), [prompt_len - 1])])
+        sane_logits(out.cpu(), "prefill")
+        times.append(time.perf_counter() - t0)
+        runner.finish(("p", r))
+    pre = sorted(times[1:])[2]
+    dec = {}
+    for b in batches:
+        ids = [("d", b, i) for i in range(b)]
+        for i in ids:
+            runner.step([StepEntry(i, toks(prompt_len), [])])
+        step = lambda: runner.step([StepEntry(i, toks(1), [0]) for i in ids])
+        for _ in range(4):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = step()
+        torch.cuda.synchronize()
+        dec[b] = (time.perf_counter() - t0) / steps
+        sane_logits(out, f"decode batch {b}")
+        for i in ids:
+            runner.finish(i)
+    return pre, dec
+
+
+def bench_design(args):
+    """``--design suripel``: prefill and decode of the Suripel design at a few real layer sizes beside the Llama
+    decoder of equal size, both with random weights through the same step function.  One JSON line."""
+    import torch
+    sizes = [int(x) for x in args.design_sizes.split(",")]
+    batches = [1, 8, 64]
+    rows = []
+    for width in sizes:
+        row = {"width": width, "layers": args.design_layers}
+        for name, cfg in (("suripel", suripel_config(width, args.design_layers)), ("llama", llama_like(width, args.design_layers))):
+            spec, runner = build_runner(cfg, args.dtype, max_tokens=66 * (args.prompt_len + 256), max_requests=64)
+            pre, dec = measure_design(runner, 32000, args.prompt_len, batches, min(args.steps, 64), seed=width)
+            row[name] = {"prefill_ms": round(pre * 1e3, 3), "prefill_tok_s": round(args.prompt_len / pre, 1),
+                         **{f"decode_b{b}_ms": round(t * 1e3, 4) for b, t in dec.items()},
+                         **{f"decode_b{b}_tok_s": round(b / t, 1) for b, t in dec.items()}}
+            log(f"width {width}, {name}: {row[name]}")
+            del runner
+            torch.cuda.empty_cache()
+        rows.append(row)
+    line = {"metric": f"prefill and decode of the Suripel design beside the Llama decoder of equal size ({args.prompt_len}-token prompts, random weights)",
+            "unit": "ms and tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "sizes": rows}
+    print(json.dumps(line), flush=True)
+    if args.record:
+        with open(args.record, "w") as f:
+            f.write(f"# bench.py --design suripel\n\nCommand:\n\n    python {' '.join(['bench.py'] + sys.argv[1:])}\n\n"
+                    f"Result (one MI355X, random weights, synthetic tokens):\n\n```json\n{json.dumps(line, indent=1)}\n```\n")
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -305,7 +404,16 @@ def main():
                     help="also write the command and the JSON line into FILE (markdown)")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="also run N requests with prompts of 128..2048 tokens and 128 decoded tokens each through the scheduler")
+    ap.add_argument("--design", default="", choices=["", "suripel"],
+                    help="instead of the serving benchmark: this design at real layer sizes beside the Llama decoder of equal size")
+    ap.add_argument("--design-sizes", default="2048,4096", metavar="LIST", help="widths of the --design models")
+    ap.add_argument("--design-layers", type=int, default=12, help="layers of the --design models")
     args = ap.parse_args()
+    if args.design:
+        if args.gpus != 1:
+            print("bench.py measures one GPU only", flush=True)
+            return 2
+        return bench_design(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported by this engine", flush=True)
         return 2
