@@ -17,7 +17,10 @@ from tiny import logit_error, prompt_ids
 pytestmark = pytest.mark.gpu
 
 # fraction of the mean logit range: (max, mean)
-TOL = {"float32": (2e-5, 2e-6), "bfloat16": (3e-2, 4e-3)}
+# (bfloat16: the matrix-core attention rounds its probabilities to 8 bits for the value product, and five
+# or six layers of recurrences pass every rounding on; the largest of some 100,000 logits strays further
+# than their mean, which is the sharper bound)
+TOL = {"float32": (2e-5, 2e-6), "bfloat16": (4e-2, 3e-3)}
 # prompt lengths (the rest of every request is given "decoded" tokens) and how many of those
 WORKLOAD = {
     "S1": ([1, 4, 23, 64, 150], 20),        # 1 and 4: shorter than the taps; 64: ends on a page of 64, 16 and 8

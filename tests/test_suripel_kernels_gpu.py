@@ -3,7 +3,6 @@
 inputs made so that a fault shows (one key that stands out just inside or just outside a window
 or a block's edge, far away, at a page's border; state rows that start as NaN)."""
 import math
-from types import SimpleNamespace
 
 import numpy as np
 import pytest
@@ -26,22 +25,14 @@ def dev(a, dtype=torch.float32):
 
 
 def step_ctx(starts, q_lens, slots, tables=()):
-    """What a step's context gives the kernels: rows of the requests one after another.
+    """A step's context as the engine makes it: rows of the requests one after another.
     ``tables``: per cache group, one list of pages per request."""
-    B = len(q_lens)
-    cu = np.concatenate([[0], np.cumsum(q_lens)])
-    pos = np.concatenate([np.arange(s, s + n) for s, n in zip(starts, q_lens)]) if B else np.zeros(0)
-    req = np.concatenate([np.full(n, b) for b, n in enumerate(q_lens)]) if B else np.zeros(0)
-    devs = []
-    for per_req in tables:
-        width = max(1, max(len(t) for t in per_req))
-        tab = np.full((B, width), -1)
-        for b, t in enumerate(per_req):
-            tab[b, :len(t)] = t
-        devs.append(dev(tab, torch.int32))
-    return SimpleNamespace(B=B, T=int(cu[-1]), q_lens=list(q_lens), max_q_len=max(q_lens), cu_q=dev(cu, torch.int32),
-                           slots=dev(slots, torch.int32), positions=dev(pos, torch.int32), req_of_token=dev(req, torch.int32),
-                           starts_dev=dev(starts, torch.int32), block_table=lambda g: devs[g])
+    from xyntetik_runner_amd.cache import RequestCache
+    from xyntetik_runner_amd.csrc.ops import load_ops
+    from xyntetik_runner_amd.engine.batch import StepContext, StepEntry
+    entries = [StepEntry(b, [0] * n, []) for b, n in enumerate(q_lens)]
+    rcs = [RequestCache(b, int(slots[b]), int(starts[b]), [list(g[b]) for g in tables], fresh=False) for b in range(len(q_lens))]
+    return StepContext(load_ops(), torch.device(DEV), entries, rcs, len(tables))
 
 
 def cuts(total, sizes):
@@ -316,6 +307,25 @@ def test_attention_random_in_portions(ops, H, G, D, Dv, size, P, page, dtype):
     got = paged_attention_case(ops, dtype, H, G, D, Dv, size, P, page, lens, plans, q, k, v, 0.3, shuffle=P)
     for b in range(3):
         close(got[b], want[b], 5e-6 if dtype == torch.float32 else 1.5e-2, f"attention request {b}")
+
+
+@pytest.mark.parametrize("H,G,D,size,P,page", [(4, 2, 64, 100, 16, 16), (8, 2, 128, 70, 32, 64), (2, 2, 32, 33, 5, 32),
+                                                 (4, 1, 16, 150, 0, 64)])
+def test_attention_on_the_matrix_cores_in_long_portions(ops, H, G, D, size, P, page):
+    """bfloat16 with head sizes the matrix-core kernels take: the window's keys go through them (row
+    blocks of a whole workgroup for the long portions, key ranges for the decoded tokens), the block
+    means through a kernel of their own, and the merge adds them."""
+    rng = np.random.default_rng(D + size)
+    lens = [420, 1, 90]
+    q = [rng.normal(size=(n, H, D)) for n in lens]
+    k = [rng.normal(size=(n, G, D)) for n in lens]
+    v = [rng.normal(size=(n, G, D)) for n in lens]
+    plans = [[(0, 300), (300, 100)] + [(i, 1) for i in range(400, 420)], [(0, 1)], cuts(90, [64, 2, 24])]
+    scale = D ** -0.5
+    want = [S.pooled_window_attention(bf16_round(qq), kk, vv, scale, size, P, cache_round=bf16_round) for qq, kk, vv in zip(q, k, v)]
+    got = paged_attention_case(ops, torch.bfloat16, H, G, D, D, size, P, page, lens, plans, q, k, v, scale, shuffle=size)
+    for b in range(3):
+        close(got[b], want[b], 1.5e-2, f"attention request {b}")
 
 
 @pytest.mark.parametrize("size,P,page", [(9, 5, 8), (12, 4, 4), (6, 16, 8), (33, 8, 16)])

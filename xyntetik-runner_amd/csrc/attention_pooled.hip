@@ -199,6 +199,74 @@ __global__ __launch_bounds__(64) void k_attention_pooled(T* __restrict__ out, co
     }
 }
 
+// ---------------------------------------------------------------- the block means alone, as a partial result
+// For the matrix-core attention kernels, which take the window's keys: the same softmax pieces
+// over the block means only, left where those kernels leave the partial result of a key range
+// (part_o [slot][kv_head][32 rows][Dv]: the normalised output; part_ml: the maximum in units of
+// log2 and the sum), so that their merge adds the two.  A record of `extras` names a block of 32
+// rows (row = token x heads-in-group + head) and its slot: request, row0, slot, q0, q_len, start.
+// One wave a row.
+template <typename T>
+__global__ __launch_bounds__(256) void k_pool_partial(float* __restrict__ part_o, float* __restrict__ part_ml,
+                                                      const T* __restrict__ q, const T* __restrict__ pk,
+                                                      const T* __restrict__ pv, const int* __restrict__ extras,
+                                                      PoolAttnArgs a) {
+    __shared__ float qs[4][AP_MAX_D];
+    const int* ex = extras + (size_t)(blockIdx.x >> 3) * 8;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = (blockIdx.x & 7) * 4 + wave;
+    const int kvh = blockIdx.y, G = a.H / a.Hk;
+    const int req = ex[0], rho = ex[1] + r, slot = ex[2], q0 = ex[3], q_len = ex[4], start = ex[5];
+    const int tok = rho / G, hg = rho - tok * G;
+    const bool row = tok < q_len;
+    if (row) {
+        const T* qrow = q + ((size_t)(q0 + tok) * a.H + kvh * G + hg) * a.D;
+        for (int d = lane; d < a.D; d += 64) qs[wave][d] = ld<T>(qrow, d);
+    }
+    __syncthreads();
+    if (!row) return;
+    const int pos = start + tok;
+    const int n_blocks = (a.P > 0 && pos - a.size + 1 > 0) ? (pos - a.size + 1) / a.P : 0;
+    float m = -INFINITY, l = 0.f;
+    float acc[AP_MAX_D / 64];
+#pragma unroll
+    for (int dd = 0; dd < AP_MAX_D / 64; ++dd) acc[dd] = 0.f;
+    if (n_blocks > 0)
+        attend_range<T>(pk, pv, a.pool_table + (size_t)req * a.pool_stride, 0, n_blocks, qs[wave], kvh, a, m, l, acc, lane);
+    const size_t at = ((size_t)slot * a.Hk + kvh) * 32 + r;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+#pragma unroll
+    for (int dd = 0; dd < AP_MAX_D / 64; ++dd) {
+        const int d = lane + 64 * dd;
+        if (d < a.Dv) part_o[at * a.Dv + d] = acc[dd] * inv;
+    }
+    if (lane == 0) {
+        part_ml[at * 2] = m * 1.44269504f;
+        part_ml[at * 2 + 1] = l;
+    }
+}
+
+extern "C" int xr_attention_pool_partial(float* part_o, float* part_ml, const void* q, const void* pk, const void* pv,
+                                         const int* extras, int n_extras, const int* pool_table, int pool_stride, int H,
+                                         int Hk, int D, int Dv, int page_size, float scale, int size, int P, int dtype,
+                                         hipStream_t stream) {
+    XR_REQUIRE(n_extras >= 0 && H > 0 && Hk > 0 && H % Hk == 0, "pooled partial: %d query heads over %d key/value heads", H, Hk);
+    XR_REQUIRE(D > 0 && D <= AP_MAX_D && Dv > 0 && Dv <= AP_MAX_D, "pooled partial: key size %d, value size %d (1 to %d)", D, Dv, AP_MAX_D);
+    const int shift = ilog2_exact(page_size);
+    XR_REQUIRE(shift >= 0, "pooled partial: page size %d is not a power of two", page_size);
+    XR_REQUIRE(size >= 1 && P >= 1 && part_o && part_ml && q && pk && pv && extras && pool_table, "pooled partial: an operand is missing");
+    if (n_extras == 0) return XR_OK;
+    PoolAttnArgs a{nullptr, nullptr, nullptr, pool_table, 0, pool_stride, H, Hk, D, Dv, shift, page_size - 1, page_size, scale, size, P};
+    dim3 grid((unsigned)n_extras * 8, Hk);
+    if (dtype == XR_F32)
+        k_pool_partial<float><<<grid, 256, 0, stream>>>(part_o, part_ml, (const float*)q, (const float*)pk, (const float*)pv, extras, a);
+    else if (dtype == XR_BF16)
+        k_pool_partial<bf16_t><<<grid, 256, 0, stream>>>(part_o, part_ml, (const bf16_t*)q, (const bf16_t*)pk, (const bf16_t*)pv, extras, a);
+    else { xr_set_error("pooled partial: bad dtype %d", dtype); return XR_BAD_ARG; }
+    XR_CHECK_LAUNCH("attention_pool_partial");
+    return XR_OK;
+}
+
 extern "C" int xr_attention_pooled(void* out, const void* q, const void* k_cache, const void* v_cache, const void* pk,
                                    const void* pv, const int* positions, const int* req_of_token, const int* block_table,
                                    int table_stride, const int* pool_table, int pool_stride, int T, int H, int Hk, int D,

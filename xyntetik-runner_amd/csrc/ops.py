@@ -66,6 +66,7 @@ _PROTOS = {
     "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_pool_blocks": [_p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_attention_pool_partial": [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
     "xr_attention_pooled": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
 }
 
@@ -772,6 +773,27 @@ class Ops:
         table = ctx.block_table(group)
         ptable = ctx.block_table(pool_group) if P else None
         out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+        if (self.use_mfma and q.dtype == torch.bfloat16 and D == Dv and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16
+                and H % Hk == 0):
+            # The window's keys go to the matrix-core kernels, every row block leaving a partial
+            # result; the block means leave theirs in a slot of their own; the kernels' merge adds them.
+            lib = self.attention_lib(D)
+            plan = ctx.attention_plan(group, H // Hk, size, Hk, page_size, extra_slot=bool(P))
+            part_o = part_ml = None
+            if plan.n_slots:
+                part_o = torch.empty((plan.n_slots, Hk, 32, D), dtype=torch.float32, device=q.device)
+                part_ml = torch.empty((plan.n_slots, Hk, 32, 2), dtype=torch.float32, device=q.device)
+            if P:
+                self.lib.check(self.lib.xr_attention_pool_partial(
+                    part_o.data_ptr(), part_ml.data_ptr(), q.data_ptr(), pk.data_ptr(), pv.data_ptr(), plan.extras.data_ptr(),
+                    plan.n_extras, ptable.data_ptr(), ptable.stride(0), H, Hk, D, Dv, page_size, float(scale), int(size),
+                    int(P), dtype_code(q.dtype), _stream()))
+            lib.check(lib.xr_attention_mfma(
+                out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
+                plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
+                ctx.starts_dev.data_ptr(), table.data_ptr(), table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
+                float(scale), int(size), _stream()))
+            return out
         self.lib.check(self.lib.xr_attention_pooled(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _ptr(pk) if P else None,
             _ptr(pv) if P else None, ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), table.data_ptr(),

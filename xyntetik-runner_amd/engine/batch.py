@@ -39,6 +39,8 @@ class AttentionPlan:
     n_jobs: int
     n_slots: int
     n_cta_items: int = 0
+    extras: Optional[torch.Tensor] = None      # [n_extras, 8] (see ``plan_attention``, ``extra_slot``)
+    n_extras: int = 0
 
 
 # The first four are the attention kernels' shapes.  The last three are tuning, not limits: they
@@ -65,11 +67,17 @@ def key_ranges(tiles: int, share: float) -> int:
 
 
 def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int,
-                   page_size: int = 64, cta_tiles: Optional[int] = None):
+                   page_size: int = 64, cta_tiles: Optional[int] = None, extra_slot: bool = False):
     """Host side of ``AttentionPlan``: ``(cta_items, items, jobs, n_slots)`` as plain Python ints.
 
     ``cta_tiles`` fixes the most tiles a 128-row item may cover (for measurements); by
     default it follows from how many such items the step has.
+
+    ``extra_slot``: every block of 32 rows gets one partial slot more than its key ranges fill,
+    for a partial result that another kernel brings (attention over entries that are no keys
+    of the cache: a layer's block means), and every item leaves a partial result for the merge.
+    A fifth value is then returned: one record ``(request, row0, slot, q0, q_len, start, 0, 0)``
+    per block of 32 rows, naming that slot.
     """
     blocks, cta_blocks = [], []
     total_tiles = 0
@@ -97,6 +105,8 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
             blocks.append(blk)
             total_tiles += blk[4]
     items, cta_items, jobs, slot = [], [], [], 0
+    extras = []
+    more = 1 if extra_slot else 0
     # longest first: workgroups are started in list order, and a long item started last
     # would run on alone at the end
     cta_blocks.sort(key=lambda blk: -blk[4])
@@ -118,9 +128,10 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
                 chunk = max(8, -(-work * n_kv_heads // ATTN_CTA_FILL))
         for b, row0, lo, hi, tiles in cta_blocks:
             parts = -(-tiles // chunk)
-            if parts <= 1:
+            if parts <= 1 and not extra_slot:
                 cta_items.append((b, row0, lo, hi, -1, q0s[b], q_lens[b], starts[b]))
                 continue
+            parts = max(1, parts)
             per = -(-tiles // parts)
             first = slot
             k = lo
@@ -133,14 +144,19 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
             rows = q_lens[b] * group_size
             for w in range(ATTN_CTA_ROWS // ATTN_ROWS):
                 if row0 + w * ATTN_ROWS < rows:
-                    jobs.append((b, row0 + w * ATTN_ROWS, first + w, n_parts, ATTN_CTA_ROWS // ATTN_ROWS, q0s[b], q_lens[b]))
+                    jobs.append((b, row0 + w * ATTN_ROWS, first + w, n_parts + more, ATTN_CTA_ROWS // ATTN_ROWS, q0s[b], q_lens[b]))
+                    if extra_slot:
+                        extras.append((b, row0 + w * ATTN_ROWS, slot + w, q0s[b], q_lens[b], starts[b], 0, 0))
+            if extra_slot:
+                slot += ATTN_CTA_ROWS // ATTN_ROWS
 
     budget = max(1, ATTN_STREAM_SLOTS // n_kv_heads)       # items that run at a time
     for b, row0, lo, hi, tiles in blocks:
         parts = 1 if len(blocks) >= budget else key_ranges(tiles, budget * tiles / total_tiles)
-        if parts <= 1:
+        if parts <= 1 and not extra_slot:
             items.append((b, row0, lo, hi, -1, q0s[b], q_lens[b], starts[b]))
             continue
+        parts = max(1, parts)
         per = -(-tiles // parts)
         first = slot
         k = lo
@@ -149,7 +165,12 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
             items.append((b, row0, k, e, slot, q0s[b], q_lens[b], starts[b]))
             slot += 1
             k = e
-        jobs.append((b, row0, first, slot - first, 1, q0s[b], q_lens[b]))
+        jobs.append((b, row0, first, slot - first + more, 1, q0s[b], q_lens[b]))
+        if extra_slot:
+            extras.append((b, row0, slot, q0s[b], q_lens[b], starts[b], 0, 0))
+            slot += 1
+    if extra_slot:
+        return cta_items, items, jobs, slot, extras
     return cta_items, items, jobs, slot
 
 
@@ -235,19 +256,23 @@ class StepContext:
         self.shared = {}        # what parts make once a step and share between layers (a rotation's table)
 
     def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
-                       page_size: int = 64) -> AttentionPlan:
+                       page_size: int = 64, extra_slot: bool = False) -> AttentionPlan:
         """The MFMA attention work list, made once per step and shared by all layers that can."""
-        key = (group_size, window, n_kv_heads, page_size)
+        key = (group_size, window, n_kv_heads, page_size, extra_slot)
         plan = self._plans.get(key)
         if plan is None:
-            cta_items, items, jobs, n_slots = plan_attention(self.starts, self.q_lens, group_size, window,
-                                                             n_kv_heads, page_size)
-            flat = [v for it in cta_items + items for v in it] + [v for j in jobs for v in j]
+            planned = plan_attention(self.starts, self.q_lens, group_size, window, n_kv_heads, page_size,
+                                     extra_slot=extra_slot)
+            cta_items, items, jobs, n_slots = planned[:4]
+            extras = planned[4] if extra_slot else []
+            flat = ([v for it in cta_items + items for v in it] + [v for j in jobs for v in j]
+                    + [v for x in extras for v in x])
             host = torch.tensor(flat, dtype=torch.int32).pin_memory()
             dev = host.to(self.device, non_blocking=True)
             nc, ni, nj = len(cta_items), len(items), len(jobs)
             nw = (nc + ni) * 8
-            plan = AttentionPlan(dev[:nw], ni, dev[nw:] if nj else None, nj, n_slots, nc)
+            plan = AttentionPlan(dev[:nw], ni, dev[nw:nw + nj * 7] if nj else None, nj, n_slots, nc,
+                                 dev[nw + nj * 7:] if extras else None, len(extras))
             plan._host = host
             self._plans[key] = plan
         return plan

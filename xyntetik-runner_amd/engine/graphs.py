@@ -70,10 +70,10 @@ class StaticDecodeContext:
         # [token_ids B][positions B][req_of_token B][cu_q B+1][seq_lens B][slots B][fresh B][starts B][want B]
         # [tables ...][plans ...]
         self._sizes = [B, B, B, B + 1, B, B, B, B, B] + [B * w for w in self.table_width]
-        self._plan_keys: List[Tuple[int, Optional[int], int]] = []
-        self._plans: Dict[Tuple[int, Optional[int], int], AttentionPlan] = {}
-        self._plan_off: Dict[Tuple[int, Optional[int], int], int] = {}
-        self._plan_splits: Dict[Tuple[int, Optional[int], int], int] = {}
+        self._plan_keys: List[Tuple[int, Optional[int], int, bool]] = []
+        self._plans: Dict[Tuple[int, Optional[int], int, bool], AttentionPlan] = {}
+        self._plan_off: Dict[Tuple[int, Optional[int], int, bool], int] = {}
+        self._plan_splits: Dict[Tuple[int, Optional[int], int, bool], int] = {}
         self._alloc()
         self.fresh_slots_host: List[int] = []
         self._copied = None
@@ -81,7 +81,7 @@ class StaticDecodeContext:
 
     def _alloc(self) -> None:
         B = self.B
-        n_plan = sum(B * self._plan_splits[k] * 8 + B * 7 for k in self._plan_keys)
+        n_plan = sum(B * self._plan_splits[k] * 8 + B * 7 + (B * 8 if k[3] else 0) for k in self._plan_keys)
         offs = np.concatenate([[0], np.cumsum(self._sizes)]).astype(np.int64)
         total = int(offs[-1]) + n_plan
         self._offs = offs
@@ -104,8 +104,13 @@ class StaticDecodeContext:
             self._plan_off[k] = base
             items = d[base:base + B * S * 8]
             jobs = d[base + B * S * 8:base + B * S * 8 + B * 7]
-            self._plans[k] = AttentionPlan(items, B * S, jobs if S > 1 else None, B if S > 1 else 0,
-                                           B * S if S > 1 else 0)
+            if k[3]:        # a slot more a request, filled by another kernel: every request has a merge job
+                extras = d[base + B * S * 8 + B * 7:base + B * S * 8 + B * 15]
+                self._plans[k] = AttentionPlan(items, B * S, jobs, B, B * (S + 1), 0, extras, B)
+                base += B * 8
+            else:
+                self._plans[k] = AttentionPlan(items, B * S, jobs if S > 1 else None, B if S > 1 else 0,
+                                               B * S if S > 1 else 0)
             base += B * S * 8 + B * 7
 
     def block_table(self, group: int) -> torch.Tensor:
@@ -117,8 +122,8 @@ class StaticDecodeContext:
                            "ctx.slots (on the device), or sets capturable = False to be run eagerly")
 
     def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
-                       page_size: int = 64) -> AttentionPlan:
-        key = (group_size, window, n_kv_heads)
+                       page_size: int = 64, extra_slot: bool = False) -> AttentionPlan:
+        key = (group_size, window, n_kv_heads, bool(extra_slot))
         if key not in self._plans:
             if torch.cuda.is_current_stream_capturing():
                 raise RuntimeError("an attention plan was first asked for during graph capture")
@@ -193,8 +198,9 @@ class StaticDecodeContext:
             self.token_ids[:n].copy_(token_source)
 
     def _fill_plan(self, h, base: int, key, starts) -> None:
-        group_size, window, _ = key
+        group_size, window, _, extra = key
         B, S = self.B, self._plan_splits[key]
+        per_req = S + 1 if extra else S         # partial slots a request
         items = h[base:base + B * S * 8].reshape(B, S, 8)
         jobs = h[base + B * S * 8:base + B * S * 8 + B * 7].reshape(B, 7)
         hi = starts.astype(np.int64) + 1                          # keys [lo, hi)
@@ -214,17 +220,26 @@ class StaticDecodeContext:
         items[:, :, 1] = 0
         items[:, :, 2] = kb
         items[:, :, 3] = ke
-        items[:, :, 4] = (np.arange(B)[:, None] * S + s_idx) if S > 1 else -1
+        items[:, :, 4] = (np.arange(B)[:, None] * per_req + s_idx) if (S > 1 or extra) else -1
         items[:, :, 5] = np.arange(B)[:, None]
         items[:, :, 6] = 1
         items[:, :, 7] = starts[:, None]
         jobs[:, 0] = np.arange(B)
         jobs[:, 1] = 0
-        jobs[:, 2] = np.arange(B) * S
-        jobs[:, 3] = S
+        jobs[:, 2] = np.arange(B) * per_req
+        jobs[:, 3] = per_req
         jobs[:, 4] = 1
         jobs[:, 5] = np.arange(B)
         jobs[:, 6] = 1
+        if extra:
+            ex = h[base + B * S * 8 + B * 7:base + B * S * 8 + B * 15].reshape(B, 8)
+            ex[:, 0] = np.arange(B)
+            ex[:, 1] = 0
+            ex[:, 2] = np.arange(B) * per_req + S
+            ex[:, 3] = np.arange(B)
+            ex[:, 4] = 1
+            ex[:, 5] = starts
+            ex[:, 6:] = 0
 
 
 class DecodeGraphs:
