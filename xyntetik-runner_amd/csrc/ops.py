@@ -58,7 +58,7 @@ _PROTOS = {
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
     "xr_layernorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
-    "xr_causal_conv": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_causal_conv": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_polynorm": [_p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rotate_rows": [_p, _p, _p, _i, _i, _i, _i, _i, _f, _p],
     "xr_gated_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _p],
@@ -627,7 +627,8 @@ class Ops:
         self.lib.check(self.lib.xr_causal_conv(out.data_ptr(), u.data_ptr(), w.data_ptr(), _ptr(state), ctx.cu_q.data_ptr(),
                                                ctx.slots.data_ptr(), ctx.req_of_token.data_ptr(), T, ctx.B, Cn, taps,
                                                u.stride(0), Cn, dtype_code(u.dtype), dtype_code(out_dtype),
-                                               1 if residual else 0, CONV_ACTIVATIONS[activation], _stream()))
+                                               1 if residual else 0, CONV_ACTIVATIONS[activation],
+                                               1 if (ctx.max_q_len == 1 and T == ctx.B) else 0, _stream()))
         return out
 
     def polynorm(self, z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
@@ -692,8 +693,11 @@ class Ops:
 
     @staticmethod
     def recurrence_state_shape(H: int, D: int, Dv: int):
-        """The per-request state of ``linear_recurrence``: S[4 j + r][c] of head h at ``[h, j, c, r]``."""
-        return (H, (D + 3) // 4, Dv, 4)
+        """The per-request state of ``linear_recurrence``: S[R j + r][c] of head h at ``[h, j, c, r]``,
+        R = the lanes that share a column in the kernel (16 for key sizes above 32, else 4; the
+        library is asked for the same numbers before every call)."""
+        R = 16 if D > 32 else 4
+        return (H, (D + R - 1) // R, Dv, R)
 
     def linear_recurrence(self, kind: str, q, k, v, state: torch.Tensor, ctx, H: int, G: int, D: int, Dv: int,
                           beta=None, gate=None, decay=None) -> torch.Tensor:
@@ -712,6 +716,10 @@ class Ops:
         T = q.shape[0]
         if tuple(q.shape) != (T, G * D) or tuple(k.shape) != (T, G * D) or tuple(v.shape) != (T, H * Dv):
             raise KernelError("linear_recurrence: view widths do not fit the heads")
+        rows, lanes = C.c_int(), C.c_int()
+        self.lib.dll.xr_recurrence_state_dims(int(D), C.byref(rows), C.byref(lanes))
+        if (H, rows.value, Dv, lanes.value) != self.recurrence_state_shape(H, D, Dv):
+            raise KernelError("linear_recurrence: the library lays its state out differently from recurrence_state_shape")
         if state.dtype != torch.float32 or tuple(state.shape[1:]) != self.recurrence_state_shape(H, D, Dv) or not state.is_contiguous():
             raise KernelError(f"linear_recurrence: state must be float32 [slots, {self.recurrence_state_shape(H, D, Dv)}]")
         if kind == "delta":

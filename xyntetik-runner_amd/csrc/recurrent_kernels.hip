@@ -3,21 +3,25 @@
 //   retention:   S <- decay_h S + k v^T;                            o = S^T q
 //   delta rule:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //
-// S is [D, Dv] and its columns never meet: column c only needs v[c], so a thread group of four
-// lanes owns one column (lane r the rows r, r+4, r+8, ...), keeps it in registers over the whole
-// portion and the two sums over D are a few fused multiply-adds and two lane exchanges a token.
-// A workgroup is 64 columns of one (request, head); queries and keys of a few tokens at a time
-// are staged in LDS, rows of a lane side by side so that they are read four at a time.
-// The same kernel runs a prompt's portion and a decoded token (a portion of one).
+// S is [D, Dv] and its columns never meet: column c only needs v[c].  A group of R adjacent lanes
+// owns one column (lane r the rows r, r+R, r+2R, ...), keeps it in registers over the whole
+// portion, and the two sums over D are a few fused multiply-adds and a sum over the group's lanes
+// (by lane permutes of the vector unit, no trip to LDS) a token.  R is 16 for key sizes above 32
+// (a token then costs a lane 3 D / 16 multiply-adds; the recurrence is a chain, so what a token
+// costs one lane is what the portion costs), else 4.  A workgroup of 256 lanes owns 256 / R
+// columns of one (request, head); queries and keys of a few tokens at a time are staged in LDS,
+// the rows of a lane side by side so that they are read four at a time.  The same kernel runs a
+// prompt's portion and a decoded token (a portion of one).
 //
-// State in memory: [slot][head][J = ceil(D/4)][Dv][4], i.e. S[4 j + r][c] at ((j * Dv) + c) * 4 + r:
-// a wave's loads and stores are contiguous.  Rows past D (when D is no multiple of 4) stay zero.
+// State in memory: [slot][head][J = ceil(D/R)][Dv][R], i.e. S[R j + r][c] at ((j * Dv) + c) * R + r:
+// a wave's loads and stores are contiguous.  Rows past D (when D is no multiple of R) stay zero.
 #include "common.h"
 
-#define REC_COLS 64          // columns of S a workgroup owns
-#define REC_TOKENS 8         // tokens staged at a time
+#define REC_TOKENS 16        // tokens staged at a time
 #define XR_REC_RETENTION 0
 #define XR_REC_DELTA 1
+
+static inline int rec_lanes(int D) { return D > 32 ? 16 : 4; }
 
 struct RecArgs {
     float* out;              // [T, H, Dv]
@@ -33,100 +37,137 @@ struct RecArgs {
     int H, G, D, Dv, ld, ld_g;   // row strides of q/k/v and of beta/gate
 };
 
-template <int MODE, int DPER>
+// the value of lane (l ^ 1), (l ^ 2) of a quad, or of the lane 4 / 8 further round a row of 16
+template <int CTRL> __device__ inline float lane_permute(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int R> __device__ inline float group_sum(float v) {
+    if (R >= 16) {
+        v += lane_permute<0x128>(v);     // row_ror:8
+        v += lane_permute<0x124>(v);     // row_ror:4
+    }
+    v += lane_permute<0x4E>(v);          // quad_perm [2,3,0,1]
+    v += lane_permute<0xB1>(v);          // quad_perm [1,0,3,2]
+    return v;
+}
+
+template <int MODE, int R, int DPER>
 __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
-    __shared__ float4 qs[REC_TOKENS][DPER];        // [token][r * (DPER/4) + j/4] as lanes read them
-    __shared__ float4 ks[REC_TOKENS][DPER];
-    __shared__ float vs[REC_TOKENS][REC_COLS];
+    constexpr int COLS = 256 / R;
+    __shared__ float4 qs[REC_TOKENS][R * DPER / 4];        // [token][r * (DPER/4) + j/4] as lanes read them
+    __shared__ float4 ks[REC_TOKENS][R * DPER / 4];
+    __shared__ float vs[REC_TOKENS][COLS];
     __shared__ float bs[REC_TOKENS], gs[REC_TOKENS];
     const int b = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
-    const int cl = tid >> 2, r = tid & 3;
-    const int col = blockIdx.x * REC_COLS + cl;
+    const int cl = tid / R, r = tid % R;
+    const int col = blockIdx.x * COLS + cl;
     const bool live = col < a.Dv;
     const int row0 = a.cu_q[b], n = a.cu_q[b + 1] - row0;
     if (n <= 0) return;
     const int kvh = h / (a.H / a.G);
-    const int J = (a.D + 3) >> 2;
-    float* sp = a.state + (((size_t)a.slots[b] * a.H + h) * J) * a.Dv * 4;
+    const int J = (a.D + R - 1) / R;
+    float* sp = a.state + (((size_t)a.slots[b] * a.H + h) * J) * a.Dv * R;
     float S[DPER];
 #pragma unroll
-    for (int j = 0; j < DPER; ++j) S[j] = (live && j < J) ? sp[((size_t)j * a.Dv + col) * 4 + r] : 0.f;
+    for (int j = 0; j < DPER; ++j) S[j] = (live && j < J) ? sp[((size_t)j * a.Dv + col) * R + r] : 0.f;
     const float dec = MODE == XR_REC_RETENTION ? a.decay[h] : 1.f;
     float* qf = reinterpret_cast<float*>(&qs[0][0]);
     float* kf = reinterpret_cast<float*>(&ks[0][0]);
 
+    // A chunk's queries, keys, values and gates go from memory into registers while the chunk before
+    // it is computed, and from there into LDS: the chain of tokens never waits for memory.
+    constexpr int NQ = REC_TOKENS * R * DPER / 256;       // staged elements of q (and of k) a lane
+    constexpr int NV = (REC_TOKENS * COLS + 255) / 256;
+    float rq[NQ], rk[NQ], rv[NV], rb = 0.f, rg = 0.f;
+    auto fetch = [&](int c0) {
+        const int nt = n - c0 < REC_TOKENS ? n - c0 : REC_TOKENS;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = tid + i * 256;
+            const int tt = idx / (R * DPER), e = idx - tt * R * DPER;
+            const int rr = e / DPER, j = e - rr * DPER, d = R * j + rr;
+            const bool ok = tt < nt && d < a.D;
+            const size_t row = (size_t)(row0 + c0 + (ok ? tt : 0)) * a.ld + (size_t)kvh * a.D + (ok ? d : 0);
+            rq[i] = ok ? a.q[row] : 0.f;
+            rk[i] = ok ? a.k[row] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = tid + i * 256;
+            const int tt = idx / COLS, c = idx - tt * COLS;
+            const int cc = blockIdx.x * COLS + c;
+            const bool ok = idx < REC_TOKENS * COLS && tt < nt && cc < a.Dv;
+            rv[i] = ok ? a.v[(size_t)(row0 + c0 + tt) * a.ld + (size_t)h * a.Dv + cc] : 0.f;
+        }
+        if (MODE == XR_REC_DELTA && tid < nt) {
+            rb = a.beta[(size_t)(row0 + c0 + tid) * a.ld_g + h];
+            rg = a.gate[(size_t)(row0 + c0 + tid) * a.ld_g + h];
+        }
+    };
+    fetch(0);
     for (int c0 = 0; c0 < n; c0 += REC_TOKENS) {
         const int nt = n - c0 < REC_TOKENS ? n - c0 : REC_TOKENS;
         __syncthreads();
-        // element d = 4 j + rr of a token goes to place rr * DPER + j; places past D hold zero
-        for (int idx = tid; idx < nt * 4 * DPER; idx += 256) {
-            const int tt = idx / (4 * DPER), e = idx - tt * 4 * DPER;
-            const int rr = e / DPER, j = e - rr * DPER, d = 4 * j + rr;
-            const size_t row = (size_t)(row0 + c0 + tt) * a.ld + (size_t)kvh * a.D;
-            qf[idx] = d < a.D ? a.q[row + d] : 0.f;
-            kf[idx] = d < a.D ? a.k[row + d] : 0.f;
-        }
-        for (int idx = tid; idx < nt * REC_COLS; idx += 256) {
-            const int tt = idx / REC_COLS, c = idx - tt * REC_COLS;
-            const int cc = blockIdx.x * REC_COLS + c;
-            vs[tt][c] = cc < a.Dv ? a.v[(size_t)(row0 + c0 + tt) * a.ld + (size_t)h * a.Dv + cc] : 0.f;
-        }
-        if (MODE == XR_REC_DELTA && tid < nt) {
-            bs[tid] = a.beta[(size_t)(row0 + c0 + tid) * a.ld_g + h];
-            gs[tid] = a.gate[(size_t)(row0 + c0 + tid) * a.ld_g + h];
-        }
+        // element d = R j + rr of a token goes to place rr * DPER + j; places past D hold zero
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) { qf[tid + i * 256] = rq[i]; kf[tid + i * 256] = rk[i]; }
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (tid + i * 256 < REC_TOKENS * COLS) (&vs[0][0])[tid + i * 256] = rv[i];
+        if (MODE == XR_REC_DELTA && tid < REC_TOKENS) { bs[tid] = rb; gs[tid] = rg; }
         __syncthreads();
+        if (c0 + REC_TOKENS < n) fetch(c0 + REC_TOKENS);
         for (int tt = 0; tt < nt; ++tt) {
             const float4* kq = &ks[tt][r * (DPER / 4)];
             const float4* qq = &qs[tt][r * (DPER / 4)];
             const float vv = vs[tt][cl];
-            float o = 0.f;
+            float4 kk[DPER / 4], q4[DPER / 4];
+#pragma unroll
+            for (int j = 0; j < DPER / 4; ++j) { kk[j] = kq[j]; q4[j] = qq[j]; }
+            float o0 = 0.f, o1 = 0.f;
             if (MODE == XR_REC_DELTA) {
                 const float g = gs[tt];
-                float dot = 0.f;
+                float d0 = 0.f, d1 = 0.f;        // two chains of sums, added at the end
 #pragma unroll
                 for (int j = 0; j < DPER; j += 4) {
-                    const float4 kk = kq[j >> 2];
                     S[j] *= g; S[j + 1] *= g; S[j + 2] *= g; S[j + 3] *= g;
-                    dot = fmaf(S[j], kk.x, dot); dot = fmaf(S[j + 1], kk.y, dot);
-                    dot = fmaf(S[j + 2], kk.z, dot); dot = fmaf(S[j + 3], kk.w, dot);
+                    d0 = fmaf(S[j], kk[j >> 2].x, d0); d1 = fmaf(S[j + 1], kk[j >> 2].y, d1);
+                    d0 = fmaf(S[j + 2], kk[j >> 2].z, d0); d1 = fmaf(S[j + 3], kk[j >> 2].w, d1);
                 }
-                dot += __shfl_xor(dot, 1, 64);
-                dot += __shfl_xor(dot, 2, 64);
-                const float u = bs[tt] * (vv - dot);
+                const float u = bs[tt] * (vv - group_sum<R>(d0 + d1));
 #pragma unroll
                 for (int j = 0; j < DPER; j += 4) {
-                    const float4 kk = kq[j >> 2];
-                    const float4 q4 = qq[j >> 2];
-                    S[j] = fmaf(kk.x, u, S[j]); S[j + 1] = fmaf(kk.y, u, S[j + 1]);
-                    S[j + 2] = fmaf(kk.z, u, S[j + 2]); S[j + 3] = fmaf(kk.w, u, S[j + 3]);
-                    o = fmaf(S[j], q4.x, o); o = fmaf(S[j + 1], q4.y, o);
-                    o = fmaf(S[j + 2], q4.z, o); o = fmaf(S[j + 3], q4.w, o);
+                    S[j] = fmaf(kk[j >> 2].x, u, S[j]); S[j + 1] = fmaf(kk[j >> 2].y, u, S[j + 1]);
+                    S[j + 2] = fmaf(kk[j >> 2].z, u, S[j + 2]); S[j + 3] = fmaf(kk[j >> 2].w, u, S[j + 3]);
+                    o0 = fmaf(S[j], q4[j >> 2].x, o0); o1 = fmaf(S[j + 1], q4[j >> 2].y, o1);
+                    o0 = fmaf(S[j + 2], q4[j >> 2].z, o0); o1 = fmaf(S[j + 3], q4[j >> 2].w, o1);
                 }
             } else {
 #pragma unroll
                 for (int j = 0; j < DPER; j += 4) {
-                    const float4 kk = kq[j >> 2];
-                    const float4 q4 = qq[j >> 2];
-                    S[j] = fmaf(dec, S[j], kk.x * vv); S[j + 1] = fmaf(dec, S[j + 1], kk.y * vv);
-                    S[j + 2] = fmaf(dec, S[j + 2], kk.z * vv); S[j + 3] = fmaf(dec, S[j + 3], kk.w * vv);
-                    o = fmaf(S[j], q4.x, o); o = fmaf(S[j + 1], q4.y, o);
-                    o = fmaf(S[j + 2], q4.z, o); o = fmaf(S[j + 3], q4.w, o);
+                    S[j] = fmaf(dec, S[j], kk[j >> 2].x * vv); S[j + 1] = fmaf(dec, S[j + 1], kk[j >> 2].y * vv);
+                    S[j + 2] = fmaf(dec, S[j + 2], kk[j >> 2].z * vv); S[j + 3] = fmaf(dec, S[j + 3], kk[j >> 2].w * vv);
+                    o0 = fmaf(S[j], q4[j >> 2].x, o0); o1 = fmaf(S[j + 1], q4[j >> 2].y, o1);
+                    o0 = fmaf(S[j + 2], q4[j >> 2].z, o0); o1 = fmaf(S[j + 3], q4[j >> 2].w, o1);
                 }
             }
-            o += __shfl_xor(o, 1, 64);
-            o += __shfl_xor(o, 2, 64);
+            const float o = group_sum<R>(o0 + o1);
             if (live && r == 0) a.out[((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col] = o;
         }
     }
     if (live) {
 #pragma unroll
         for (int j = 0; j < DPER; ++j)
-            if (j < J) sp[((size_t)j * a.Dv + col) * 4 + r] = S[j];
+            if (j < J) sp[((size_t)j * a.Dv + col) * R + r] = S[j];
     }
 }
 
-extern "C" int xr_state_rows_per_head(int D) { return (D + 3) / 4; }
+// the shape of a request's state as [H, shape[0], Dv, shape[1]]
+extern "C" int xr_recurrence_state_dims(int D, int* rows, int* lanes) {
+    *lanes = rec_lanes(D);
+    *rows = (D + *lanes - 1) / *lanes;
+    return XR_OK;
+}
 
 extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, const float* v, const float* beta,
                                     const float* gate, const float* decay, float* state, const int* cu_q,
@@ -140,14 +181,14 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
     XR_REQUIRE(out && q && k && v && state && cu_q && slots, "recurrence: a pointer is missing");
     if (B == 0) return XR_OK;
     RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g};
-    dim3 grid((Dv + REC_COLS - 1) / REC_COLS, H, B);
-    const int per = (D + 3) / 4;
+    const int R = rec_lanes(D), cols = 256 / R, per = (D + R - 1) / R;
+    dim3 grid((Dv + cols - 1) / cols, H, B);
 #define REC(M)                                                                          \
     do {                                                                                \
-        if (per <= 8) k_recurrence<M, 8><<<grid, 256, 0, stream>>>(a);                  \
-        else if (per <= 16) k_recurrence<M, 16><<<grid, 256, 0, stream>>>(a);           \
-        else if (per <= 32) k_recurrence<M, 32><<<grid, 256, 0, stream>>>(a);           \
-        else k_recurrence<M, 64><<<grid, 256, 0, stream>>>(a);                          \
+        if (R == 4) k_recurrence<M, 4, 8><<<grid, 256, 0, stream>>>(a);                 \
+        else if (per <= 4) k_recurrence<M, 16, 4><<<grid, 256, 0, stream>>>(a);         \
+        else if (per <= 8) k_recurrence<M, 16, 8><<<grid, 256, 0, stream>>>(a);         \
+        else k_recurrence<M, 16, 16><<<grid, 256, 0, stream>>>(a);                      \
     } while (0)
     if (mode == XR_REC_DELTA) REC(XR_REC_DELTA);
     else REC(XR_REC_RETENTION);

@@ -10,33 +10,39 @@
 
 // ---------------------------------------------------------------- layer norm
 // y = (x - mean) / sqrt(var + eps) * w, var = mean((x - mean)^2); no bias.  One workgroup a row.
-__device__ inline float block_sum_256(float v, float* part) {
+// NW waves a row: 4 where there are rows enough to fill the chip, 16 for the few rows of a
+// decode step, whose time is the latency of one workgroup's passes over its row.
+template <int NW> __device__ inline float block_sum(float v, float* part) {
     v = wave_sum(v);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = v;
     __syncthreads();
-    return part[0] + part[1] + part[2] + part[3];
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) t += part[i];
+    return t;
 }
+#define FEW_ROWS 128
 
-template <typename TO>
-__global__ __launch_bounds__(256) void k_layernorm(TO* __restrict__ out, const float* __restrict__ x,
-                                                   const float* __restrict__ w, const int* __restrict__ rows,
-                                                   int E, int ldx, float eps) {
-    __shared__ float part[4];
+template <typename TO, int NW>
+__global__ __launch_bounds__(64 * NW) void k_layernorm(TO* __restrict__ out, const float* __restrict__ x,
+                                                      const float* __restrict__ w, const int* __restrict__ rows,
+                                                      int E, int ldx, float eps) {
+    __shared__ float part[NW];
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     const float* xr = x + (size_t)src * ldx;
     float s = 0.f;
-    for (int i = threadIdx.x; i < E; i += 256) s += xr[i];
-    const float mean = block_sum_256(s, part) / (float)E;
+    for (int i = threadIdx.x; i < E; i += 64 * NW) s += xr[i];
+    const float mean = block_sum<NW>(s, part) / (float)E;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < E; i += 256) {
+    for (int i = threadIdx.x; i < E; i += 64 * NW) {
         const float d = xr[i] - mean;
         ss += d * d;
     }
-    const float rinv = 1.0f / sqrtf(block_sum_256(ss, part) / (float)E + eps);
+    const float rinv = 1.0f / sqrtf(block_sum<NW>(ss, part) / (float)E + eps);
     TO* o = out + (size_t)r * E;
-    for (int i = threadIdx.x; i < E; i += 256) st<TO>(o, i, (xr[i] - mean) * rinv * (w ? w[i] : 1.f));
+    for (int i = threadIdx.x; i < E; i += 64 * NW) st<TO>(o, i, (xr[i] - mean) * rinv * (w ? w[i] : 1.f));
 }
 
 extern "C" int xr_layernorm(void* out, const float* x, const float* w, const int* rows, int R, int E, int ldx,
@@ -45,8 +51,14 @@ extern "C" int xr_layernorm(void* out, const float* x, const float* w, const int
     XR_REQUIRE(eps >= 0.f, "layernorm: eps %g is negative", eps);
     XR_REQUIRE(out_dtype == XR_F32 || out_dtype == XR_BF16, "layernorm: bad dtype %d", out_dtype);
     if (R == 0) return XR_OK;
-    if (out_dtype == XR_F32) k_layernorm<float><<<R, 256, 0, stream>>>((float*)out, x, w, rows, E, ldx, eps);
-    else k_layernorm<bf16_t><<<R, 256, 0, stream>>>((bf16_t*)out, x, w, rows, E, ldx, eps);
+    const bool few = R <= FEW_ROWS && E >= 1024;
+    if (out_dtype == XR_F32) {
+        if (few) k_layernorm<float, 16><<<R, 1024, 0, stream>>>((float*)out, x, w, rows, E, ldx, eps);
+        else k_layernorm<float, 4><<<R, 256, 0, stream>>>((float*)out, x, w, rows, E, ldx, eps);
+    } else {
+        if (few) k_layernorm<bf16_t, 16><<<R, 1024, 0, stream>>>((bf16_t*)out, x, w, rows, E, ldx, eps);
+        else k_layernorm<bf16_t, 4><<<R, 256, 0, stream>>>((bf16_t*)out, x, w, rows, E, ldx, eps);
+    }
     XR_CHECK_LAUNCH("layernorm");
     return XR_OK;
 }
@@ -55,29 +67,32 @@ extern "C" int xr_layernorm(void* out, const float* x, const float* w, const int
 // y_t[c] = sum_j w[c][j] * u_(t - taps + 1 + j)[c]  (+ u_t[c] with `residual`), then the activation.
 // Inputs before a portion's first row come from the request's state row, which holds its last
 // taps - 1 inputs, oldest first, and is zero for a request that begins.  The state is rewritten by
-// a second kernel once every row has been read.
+// a second kernel once every row has been read; in a step where every request brings one row
+// (`fuse`) a row's own thread is the only one that reads its request's state and rewrites it itself.
 #define CONV_MAX_TAPS 16
 #define XR_CONV_NONE 0
 #define XR_CONV_SILU 1
 
 template <typename TU, typename TO>
 __global__ __launch_bounds__(256) void k_causal_conv(TO* __restrict__ out, const TU* __restrict__ u,
-                                                     const float* __restrict__ w, const TU* __restrict__ state,
+                                                     const float* __restrict__ w, TU* state,
                                                      const int* __restrict__ cu_q, const int* __restrict__ slots,
                                                      const int* __restrict__ req_of_token, int C, int taps, int ld_u,
-                                                     int ld_out, int residual, int act) {
+                                                     int ld_out, int residual, int act, int fuse) {
     const int t = blockIdx.y;
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
     const int b = req_of_token[t];
     const int row0 = cu_q[b];
     const int i = t - row0;
-    const TU* srow = state + (size_t)slots[b] * (taps - 1) * C;
+    TU* srow = state + (size_t)slots[b] * (taps - 1) * C;
     float acc = 0.f;
     for (int j = 0; j < taps; ++j) {
         const int s = i - (taps - 1) + j;
         const float val = s >= 0 ? ld<TU>(u, (size_t)(row0 + s) * ld_u + c) : ld<TU>(srow, (size_t)(taps - 1 + s) * C + c);
         acc = fmaf(w[(size_t)c * taps + j], val, acc);
+        // one row a request: input j of this row is state entry j, which moves one place down
+        if (fuse && j > 0) st<TU>(srow, (size_t)(j - 1) * C + c, val);
     }
     if (residual) acc += ld<TU>(u, (size_t)t * ld_u + c);
     if (act == XR_CONV_SILU) acc = acc / (1.0f + expf(-acc));
@@ -110,20 +125,22 @@ __global__ __launch_bounds__(256) void k_conv_state(TU* __restrict__ state, cons
 
 extern "C" int xr_causal_conv(void* out, const void* u, const float* w, void* state, const int* cu_q, const int* slots,
                               const int* req_of_token, int T, int B, int C, int taps, int ld_u, int ld_out,
-                              int u_dtype, int out_dtype, int residual, int act, hipStream_t stream) {
+                              int u_dtype, int out_dtype, int residual, int act, int one_row_each, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && B >= 0 && C > 0 && ld_u >= C && ld_out >= C, "causal_conv: bad sizes T=%d B=%d C=%d ld_u=%d ld_out=%d",
                T, B, C, ld_u, ld_out);
     XR_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "causal_conv: %d taps (1 to %d)", taps, CONV_MAX_TAPS);
     XR_REQUIRE(act == XR_CONV_NONE || act == XR_CONV_SILU, "causal_conv: activation code %d", act);
     XR_REQUIRE(out != u, "causal_conv: the result cannot overwrite its input");
     XR_REQUIRE(taps == 1 || state != nullptr, "causal_conv: a convolution of %d taps needs its state", taps);
+    XR_REQUIRE(!one_row_each || T == B, "causal_conv: %d rows of %d requests are not one row each", T, B);
     if (T == 0 || B == 0) return XR_OK;
+    const int fuse = one_row_each && taps > 1 ? 1 : 0;
     dim3 grid((C + 255) / 256, T), sgrid((C + 255) / 256, B);
 #define CC(TU, TO)                                                                                                   \
     do {                                                                                                             \
-        k_causal_conv<TU, TO><<<grid, 256, 0, stream>>>((TO*)out, (const TU*)u, w, (const TU*)state, cu_q, slots,     \
-                                                        req_of_token, C, taps, ld_u, ld_out, residual, act);          \
-        if (taps > 1) k_conv_state<TU><<<sgrid, 256, 0, stream>>>((TU*)state, (const TU*)u, cu_q, slots, C, taps, ld_u); \
+        k_causal_conv<TU, TO><<<grid, 256, 0, stream>>>((TO*)out, (const TU*)u, w, (TU*)state, cu_q, slots,           \
+                                                        req_of_token, C, taps, ld_u, ld_out, residual, act, fuse);    \
+        if (taps > 1 && !fuse) k_conv_state<TU><<<sgrid, 256, 0, stream>>>((TU*)state, (const TU*)u, cu_q, slots, C, taps, ld_u); \
     } while (0)
     if (u_dtype == XR_F32 && out_dtype == XR_F32) CC(float, float);
     else if (u_dtype == XR_F32 && out_dtype == XR_BF16) CC(float, bf16_t);
@@ -138,25 +155,25 @@ extern "C" int xr_causal_conv(void* out, const void* u, const float* w, void* st
 // ---------------------------------------------------------------- PolyNorm
 // y = a N(z) + b N(z^2) + c N(z^3) + e, powers element by element, N(v) = v / sqrt(mean(v^2) + eps)
 // over the row.  One workgroup a row: the three sums in one pass, the result in a second.
-template <typename TZ, typename TO>
-__global__ __launch_bounds__(256) void k_polynorm(TO* __restrict__ out, const TZ* __restrict__ z,
-                                                  const float* __restrict__ coef, int F, int ld_z, float eps) {
-    __shared__ float part[4];
+template <typename TZ, typename TO, int NW>
+__global__ __launch_bounds__(64 * NW) void k_polynorm(TO* __restrict__ out, const TZ* __restrict__ z,
+                                                     const float* __restrict__ coef, int F, int ld_z, float eps) {
+    __shared__ float part[NW];
     const TZ* zr = z + (size_t)blockIdx.x * ld_z;
     float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-    for (int i = threadIdx.x; i < F; i += 256) {
+    for (int i = threadIdx.x; i < F; i += 64 * NW) {
         const float v = ld<TZ>(zr, i), v2 = v * v, v3 = v2 * v;
         s2 += v2;
         s4 += v2 * v2;
         s6 += v3 * v3;
     }
     const float inv = 1.0f / (float)F;
-    const float r1 = coef[0] / sqrtf(block_sum_256(s2, part) * inv + eps);
-    const float r2 = coef[1] / sqrtf(block_sum_256(s4, part) * inv + eps);
-    const float r3 = coef[2] / sqrtf(block_sum_256(s6, part) * inv + eps);
+    const float r1 = coef[0] / sqrtf(block_sum<NW>(s2, part) * inv + eps);
+    const float r2 = coef[1] / sqrtf(block_sum<NW>(s4, part) * inv + eps);
+    const float r3 = coef[2] / sqrtf(block_sum<NW>(s6, part) * inv + eps);
     const float e = coef[3];
     TO* o = out + (size_t)blockIdx.x * F;
-    for (int i = threadIdx.x; i < F; i += 256) {
+    for (int i = threadIdx.x; i < F; i += 64 * NW) {
         const float v = ld<TZ>(zr, i), v2 = v * v;
         st<TO>(o, i, v * r1 + v2 * r2 + v2 * v * r3 + e);
     }
@@ -166,10 +183,17 @@ extern "C" int xr_polynorm(void* out, const void* z, const float* coef, int T, i
                            int out_dtype, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && F > 0 && ld_z >= F, "polynorm: bad sizes T=%d F=%d ld=%d", T, F, ld_z);
     if (T == 0) return XR_OK;
-    if (z_dtype == XR_F32 && out_dtype == XR_F32) k_polynorm<float, float><<<T, 256, 0, stream>>>((float*)out, (const float*)z, coef, F, ld_z, eps);
-    else if (z_dtype == XR_F32 && out_dtype == XR_BF16) k_polynorm<float, bf16_t><<<T, 256, 0, stream>>>((bf16_t*)out, (const float*)z, coef, F, ld_z, eps);
-    else if (z_dtype == XR_BF16 && out_dtype == XR_BF16) k_polynorm<bf16_t, bf16_t><<<T, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)z, coef, F, ld_z, eps);
+    const bool few = T <= FEW_ROWS && F >= 1024;
+#define PN(TZ, TO)                                                                                                        \
+    do {                                                                                                                  \
+        if (few) k_polynorm<TZ, TO, 16><<<T, 1024, 0, stream>>>((TO*)out, (const TZ*)z, coef, F, ld_z, eps);              \
+        else k_polynorm<TZ, TO, 4><<<T, 256, 0, stream>>>((TO*)out, (const TZ*)z, coef, F, ld_z, eps);                    \
+    } while (0)
+    if (z_dtype == XR_F32 && out_dtype == XR_F32) PN(float, float);
+    else if (z_dtype == XR_F32 && out_dtype == XR_BF16) PN(float, bf16_t);
+    else if (z_dtype == XR_BF16 && out_dtype == XR_BF16) PN(bf16_t, bf16_t);
     else { xr_set_error("polynorm: bad dtypes %d %d", z_dtype, out_dtype); return XR_BAD_ARG; }
+#undef PN
     XR_CHECK_LAUNCH("polynorm");
     return XR_OK;
 }
