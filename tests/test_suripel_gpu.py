@@ -4,6 +4,10 @@ batches in pools so small that pages and state slots are used again, long decodi
 recorded steps, and greedy generation through the engine's own entry point and scheduler.
 Three configurations that differ in every size and constant (``suripel_tiny``)."""
 import io
+import json
+import os
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -159,6 +163,45 @@ def test_greedy_generation_through_the_entry_point(models, which):
     got = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=8))
     assert got == wanted
     assert llm.runner.manager.all_free()
+
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_command_line(models):
+    d, cfg, w, *_ = models["S2"]
+    prompt = prompt_ids(9, cfg["vocab"], 21)
+    wanted = S.greedy(cfg, w, prompt, 5)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "runner"), "-m", d, "--ids", ",".join(map(str, prompt)), "-n", "5",
+           "--temp", "0", "--dtype", "float32", "-c", "128", "-b", "4"]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stderr
+    assert p.stdout.strip() == ",".join(map(str, prompt + wanted))
+    # sampling with a seed: the same tokens twice, other tokens with another seed or none of them equal by luck alone
+    cmd = cmd[:6] + ["-n", "12", "--temp", "1.3", "--top-k", "20", "--dtype", "float32", "-c", "128", "-s"]
+    a = subprocess.run(cmd + ["5"], capture_output=True, text=True, timeout=120)
+    b = subprocess.run(cmd + ["5"], capture_output=True, text=True, timeout=120)
+    c = subprocess.run(cmd + ["6"], capture_output=True, text=True, timeout=120)
+    assert a.returncode == 0 and a.stdout == b.stdout and a.stdout != c.stdout
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(models, tmp_path, dtype):
+    """bin/trace_run as a user runs it: a child process, steps on stdin, 'done <step>' lines back,
+    four state slots and pools for the tokens that are live."""
+    d, cfg, w, reqs, plens, want = models["S3"]
+    steps = traces.mixed(reqs, plens, max_live=4, seed=2)
+    out = str(tmp_path / "out")
+    p = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", dtype,
+                          "--out", out, "--max-tokens", str(traces.max_live_tokens(steps, 64))],
+                         stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    for st in steps:
+        p.stdin.write(json.dumps(st) + "\n")
+        p.stdin.flush()
+        assert p.stdout.readline().strip() == f"done {st['step']}"
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
+    check(traces.collect(steps, out, cfg["vocab"]), want, dtype, "trace_run")
 
 
 def test_model_is_built_from_its_config(models):

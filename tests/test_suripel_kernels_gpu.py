@@ -144,6 +144,33 @@ def test_causal_conv_in_portions_and_batches(ops, taps, residual, act):
         close(got[b], want[b], 3e-6, f"conv request {b}")
 
 
+@pytest.mark.parametrize("E,taps", [(48, 3), (1100, 4), (64, 1)])
+def test_norm_and_convolution_in_one_kernel_for_steps_of_one_row(ops, E, taps):
+    """Five requests decode 9 tokens each, one row a request and step: the fused kernel against
+    the plain layer norm and convolution over each request's whole sequence, and bit for bit
+    against the two kernels it stands for."""
+    rng = np.random.default_rng(E)
+    B, n = 5, 9
+    xs = rng.normal(size=(B, n, E)) * 2 + 0.3
+    w, cw = rng.normal(size=E), rng.normal(size=(E, taps))
+    want = []
+    for b in range(B):
+        h = S.layer_norm(xs[b], w, 1e-5)
+        want.append(h + S.causal_conv(h, cw))
+    mk = lambda: torch.zeros((B + 1, taps - 1, E), device=DEV) if taps > 1 else None
+    st_a, st_b = mk(), mk()
+    slots = [3, 0, 4, 1, 2]
+    for t in range(n):
+        ctx = step_ctx([t] * B, [1] * B, slots)
+        x = dev(xs[:, t])
+        got = ops.layernorm_conv(x, dev(w), 1e-5, dev(cw), st_a, ctx, torch.float32)
+        two = ops.causal_conv(ops.layernorm(x, dev(w), 1e-5, torch.float32), dev(cw), st_b, ctx, torch.float32, residual=True)
+        assert torch.equal(got, two)
+        if taps > 1:
+            assert torch.equal(st_a, st_b)
+        close(got.cpu(), np.stack([want[b][t] for b in range(B)]), 3e-6, f"token {t}")
+
+
 # ----------------------------------------------------------------------------- recurrences
 def run_recurrence(ops, kind, qs, ks, vs, extra, H, G, D, Dv, plans, slots, n_slots):
     """Requests (lists of per-token arrays) through ``linear_recurrence`` in the given portions."""

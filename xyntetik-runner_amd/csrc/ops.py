@@ -58,6 +58,7 @@ _PROTOS = {
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
     "xr_layernorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
+    "xr_layernorm_conv": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _p],
     "xr_causal_conv": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_polynorm": [_p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rotate_rows": [_p, _p, _p, _i, _i, _i, _i, _i, _f, _p],
@@ -629,6 +630,31 @@ class Ops:
                                                u.stride(0), Cn, dtype_code(u.dtype), dtype_code(out_dtype),
                                                1 if residual else 0, CONV_ACTIVATIONS[activation],
                                                1 if (ctx.max_q_len == 1 and T == ctx.B) else 0, _stream()))
+        return out
+
+    def layernorm_conv(self, x: torch.Tensor, w: Optional[torch.Tensor], eps: float, conv_w: torch.Tensor,
+                       state: Optional[torch.Tensor], ctx, out_dtype: torch.dtype) -> torch.Tensor:
+        """``h + conv(h)`` with ``h = layernorm(x)`` in one kernel, for a step in which every request
+        brings one row (row b of ``x`` is request b's): the same result as ``layernorm`` in 32 bits
+        followed by ``causal_conv`` with ``residual``, and the same update of ``state``."""
+        self._dev(x, w, conv_w, state)
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+            raise KernelError("layernorm_conv input must be float32 [rows, width] with unit column stride")
+        R, E = x.shape
+        if ctx.max_q_len != 1 or R != ctx.B:
+            raise KernelError("layernorm_conv is for steps of one row a request")
+        if w is not None and (w.dtype != torch.float32 or w.numel() != E or not w.is_contiguous()):
+            raise KernelError(f"layernorm_conv: the norm's weight must be float32 [{E}]")
+        if conv_w.dtype != torch.float32 or conv_w.dim() != 2 or conv_w.shape[0] != E or not conv_w.is_contiguous():
+            raise KernelError(f"layernorm_conv: the convolution's weight must be float32 [{E}, taps]")
+        taps = conv_w.shape[1]
+        if taps > 1 and (state is None or state.dtype != torch.float32 or tuple(state.shape[1:]) != (taps - 1, E)
+                         or not state.is_contiguous()):
+            raise KernelError(f"layernorm_conv state must be float32 [slots, {taps - 1}, {E}]")
+        out = torch.empty((R, E), dtype=out_dtype, device=x.device)
+        self.lib.check(self.lib.xr_layernorm_conv(out.data_ptr(), x.data_ptr(), _ptr(w), conv_w.data_ptr(), _ptr(state),
+                                                  ctx.slots.data_ptr(), R, E, x.stride(0), taps, float(eps),
+                                                  dtype_code(out_dtype), _stream()))
         return out
 
     def polynorm(self, z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:

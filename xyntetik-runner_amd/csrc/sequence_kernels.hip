@@ -152,6 +152,62 @@ extern "C" int xr_causal_conv(void* out, const void* u, const float* w, void* st
     return XR_OK;
 }
 
+// Layer norm and the convolution behind it in one kernel, for a step in which every request
+// brings one row: row b is request b's, its convolution reads the request's carried inputs and
+// the row itself, and the thread that owns a channel moves that channel's carried inputs on.
+//   h = layernorm(x);  y = h + sum_j cw[:, j] * (carried_j, ..., h);  carried <- (carried_1.., h)
+template <typename TO, int NW>
+__global__ __launch_bounds__(64 * NW) void k_layernorm_conv(TO* __restrict__ out, const float* __restrict__ x,
+                                                           const float* __restrict__ w, const float* __restrict__ cw,
+                                                           float* state, const int* __restrict__ slots, int E, int ldx,
+                                                           int taps, float eps) {
+    __shared__ float part[NW];
+    const int r = blockIdx.x;
+    const float* xr = x + (size_t)r * ldx;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < E; i += 64 * NW) s += xr[i];
+    const float mean = block_sum<NW>(s, part) / (float)E;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < E; i += 64 * NW) {
+        const float d = xr[i] - mean;
+        ss += d * d;
+    }
+    const float rinv = 1.0f / sqrtf(block_sum<NW>(ss, part) / (float)E + eps);
+    float* srow = state + (size_t)slots[r] * (taps - 1) * E;
+    TO* o = out + (size_t)r * E;
+    for (int i = threadIdx.x; i < E; i += 64 * NW) {
+        const float h = (xr[i] - mean) * rinv * (w ? w[i] : 1.f);
+        float acc = 0.f;
+        for (int j = 0; j < taps - 1; ++j) {
+            const float val = srow[(size_t)j * E + i];
+            acc = fmaf(cw[(size_t)i * taps + j], val, acc);
+            if (j > 0) srow[(size_t)(j - 1) * E + i] = val;
+        }
+        acc = fmaf(cw[(size_t)i * taps + taps - 1], h, acc);
+        if (taps > 1) srow[(size_t)(taps - 2) * E + i] = h;
+        st<TO>(o, i, acc + h);
+    }
+}
+
+extern "C" int xr_layernorm_conv(void* out, const float* x, const float* w, const float* cw, float* state,
+                                 const int* slots, int R, int E, int ldx, int taps, float eps, int out_dtype,
+                                 hipStream_t stream) {
+    XR_REQUIRE(R >= 0 && E > 0 && ldx >= E, "layernorm_conv: bad sizes R=%d E=%d ldx=%d", R, E, ldx);
+    XR_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS && cw && slots && (taps == 1 || state), "layernorm_conv: %d taps, or an operand is missing", taps);
+    XR_REQUIRE(out_dtype == XR_F32 || out_dtype == XR_BF16, "layernorm_conv: bad dtype %d", out_dtype);
+    if (R == 0) return XR_OK;
+    const bool few = R <= FEW_ROWS && E >= 1024;
+    if (out_dtype == XR_F32) {
+        if (few) k_layernorm_conv<float, 16><<<R, 1024, 0, stream>>>((float*)out, x, w, cw, state, slots, E, ldx, taps, eps);
+        else k_layernorm_conv<float, 4><<<R, 256, 0, stream>>>((float*)out, x, w, cw, state, slots, E, ldx, taps, eps);
+    } else {
+        if (few) k_layernorm_conv<bf16_t, 16><<<R, 1024, 0, stream>>>((bf16_t*)out, x, w, cw, state, slots, E, ldx, taps, eps);
+        else k_layernorm_conv<bf16_t, 4><<<R, 256, 0, stream>>>((bf16_t*)out, x, w, cw, state, slots, E, ldx, taps, eps);
+    }
+    XR_CHECK_LAUNCH("layernorm_conv");
+    return XR_OK;
+}
+
 // ---------------------------------------------------------------- PolyNorm
 // y = a N(z) + b N(z^2) + c N(z^3) + e, powers element by element, N(v) = v / sqrt(mean(v^2) + eps)
 // over the row.  One workgroup a row: the three sums in one pass, the result in a second.

@@ -57,15 +57,19 @@ class FilteredPreNormBlock(Block):
     filter_names = ("mixer_filter", "feed_forward_filter")
     needs_feed_forward = None       # with or without; the second norm and filter then do nothing
 
+    def _read(self, ctx, cache, x, norm: str, flt: str):
+        """What a sublayer reads: the norm of ``x`` through the filter, in one kernel if the filter has one."""
+        f, state = self.filters[flt], cache.states.get(flt)
+        fused = getattr(f, "forward_normed", None)
+        h = fused(ctx, state, x, self.norms[norm]) if fused is not None else None
+        if h is None:
+            h = f.forward(ctx, state, self.norms[norm].forward(ctx, x))
+        return h
+
     def forward(self, ctx, cache, x):
-        h = self.norms["mixer_norm"].forward(ctx, x)
-        h = self.filters["mixer_filter"].forward(ctx, cache.states.get("mixer_filter"), h)
-        self.mixer.forward_add(ctx, cache, h, x)
-        if self.feed_forward is None:
-            return
-        h = self.norms["feed_forward_norm"].forward(ctx, x)
-        h = self.filters["feed_forward_filter"].forward(ctx, cache.states.get("feed_forward_filter"), h)
-        self.feed_forward.forward_add(ctx, h, x)
+        self.mixer.forward_add(ctx, cache, self._read(ctx, cache, x, "mixer_norm", "mixer_filter"), x)
+        if self.feed_forward is not None:
+            self.feed_forward.forward_add(ctx, self._read(ctx, cache, x, "feed_forward_norm", "feed_forward_filter"), x)
 
     def state_specs(self):
         out = super().state_specs()

@@ -47,4 +47,15 @@ class CausalConv(SequenceFilter):
                                        activation=self.activation)
 
 
+    def forward_normed(self, ctx, state, x, norm):
+        """``forward(ctx, state, norm.forward(ctx, x))`` in one kernel where there is one: a step of one
+        row a request, a layer norm in front, the input added, no activation.  None: the caller
+        runs the two one after the other."""
+        from .norm import LayerNorm
+        if (ctx.max_q_len != 1 or not isinstance(norm, LayerNorm) or not self.residual or self.activation is not None
+                or self.weight is None):
+            return None
+        return self.rt.ops.layernorm_conv(x, norm.weight, norm.eps, self.weight, state, ctx, self.rt.dtype)
+
+
 register_filter("causal_conv", CausalConv)
