@@ -134,10 +134,11 @@ def attention_mixer(h, w, p, m, kv=None):
     has none of its own.  Returns (output, (keys, values) as a cache would hold them)."""
     T = h.shape[0]
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = causal_conv(h @ w[p + "q"].T, w[p + "q.conv"]).reshape(T, H, D)
+    conv = (lambda u, name: causal_conv(u, w[p + name + ".conv"])) if m.get("conv") else (lambda u, name: u)
+    q = conv(h @ w[p + "q"].T, "q").reshape(T, H, D)
     if kv is None:
-        k = causal_conv(h @ w[p + "k"].T, w[p + "k.conv"]).reshape(T, G, D)
-        v = causal_conv(h @ w[p + "v"].T, w[p + "v.conv"]).reshape(T, G, Dv)
+        k = conv(h @ w[p + "k"].T, "k").reshape(T, G, D)
+        v = conv(h @ w[p + "v"].T, "v").reshape(T, G, Dv)
     else:
         k, v = kv
     o = pooled_window_attention(q, k, v, m["scale"], m["mask"]["size"], m["mask"].get("pool", 0))
@@ -168,9 +169,10 @@ def gated_delta_rule(q, k, v, beta, g):
 def delta_mixer(h, w, p, m, eps):
     T = h.shape[0]
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = silu(causal_conv(h @ w[p + "q"].T, w[p + "q.conv"])).reshape(T, G, D)
-    k = silu(causal_conv(h @ w[p + "k"].T, w[p + "k.conv"])).reshape(T, G, D)
-    v = silu(causal_conv(h @ w[p + "v"].T, w[p + "v.conv"])).reshape(T, H, Dv)
+    conv = (lambda u, name: causal_conv(u, w[p + name + ".conv"])) if m.get("conv") else (lambda u, name: u)
+    q = silu(conv(h @ w[p + "q"].T, "q")).reshape(T, G, D)
+    k = silu(conv(h @ w[p + "k"].T, "k")).reshape(T, G, D)
+    v = silu(conv(h @ w[p + "v"].T, "v")).reshape(T, H, Dv)
     q = unit(q) * D ** -0.5
     k = unit(k)
     per = H // G

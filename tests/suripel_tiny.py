@@ -15,13 +15,18 @@ def attention(heads, kv_heads, dim, vdim, size, pool, conv, scale, kv_from=None)
          "mask": {"size": size, "pool": pool}}
     if not pool:
         del m["mask"]["pool"]
+    if not conv:
+        del m["conv"]               # no convolution of the projections, and no tensors of one
     if kv_from is not None:
         m["kv_from"] = kv_from
     return {"type": "attention", "mixer": m}
 
 
 def delta(heads, kv_heads, dim, vdim, conv):
-    return {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}}
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+    if not conv:
+        del m["conv"]
+    return {"type": "delta", "mixer": m}
 
 
 def retention(heads, dim, vdim, decay, rot=None):
@@ -52,15 +57,15 @@ TINY_S1 = {
 }
 
 # attention first; a block longer than the window; attention without blocks; convolutions of one
-# tap; key sizes that are no multiples of 4; heads = key heads in attention, one key head in delta
+# tap and mixers without any; key sizes that are no multiples of 4; heads = key heads in attention, one key head in delta
 TINY_S2 = {
     "architecture": "Suripel", "vocab": 97, "width": 40, "norm": {"eps": 1e-6}, "canon": {"taps": 2},
     "layers": [
         with_ff(attention(2, 2, 10, 10, 4, 8, 1, 0.4), 64),
         with_ff(delta(3, 1, 7, 9, 4), 48),
-        with_ff(attention(3, 1, 8, 6, 11, 0, 4, 0.25), 64),
+        with_ff(attention(3, 1, 8, 6, 11, 0, 0, 0.25), 64),
         with_ff(retention(2, 6, 5, [0.5, 0.9375], rot=(6, 10000.0)), 32),
-        with_ff(delta(2, 2, 16, 16, 1), 48),
+        with_ff(delta(2, 2, 16, 16, 0), 48),
     ],
 }
 

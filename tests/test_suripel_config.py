@@ -35,7 +35,8 @@ def test_parts_get_their_constants_from_the_config():
     _, cfg, spec = build(TINY_S2)
     m = spec.layers[0].mixer
     assert m.kind == "pooled_window_attention" and m.params["window"] == 4 and m.params["pool"] == 8 and m.params["keep"] == 8
-    assert spec.layers[2].mixer.params["pool"] == 0 and spec.layers[2].mixer.params["conv_taps"] == 4
+    assert spec.layers[2].mixer.params["pool"] == 0 and spec.layers[2].mixer.params["conv_taps"] == 0
+    assert spec.layers[0].mixer.params["conv_taps"] == 1 and spec.layers[4].mixer.params["conv_taps"] == 0
     assert spec.layers[1].mixer.kind == "gated_delta" and spec.layers[1].mixer.params["num_kv_heads"] == 1
     assert spec.layers[3].mixer.params["position"].params == {"head_dim": 6, "theta": 10000.0, "rotary_dim": 6}
     assert spec.layers[0].filters["mixer_filter"].params["taps"] == 2

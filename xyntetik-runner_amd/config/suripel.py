@@ -32,7 +32,7 @@ class SuripelMixer:
     kv_heads: int
     dim: int
     vdim: int
-    conv: int = 1                       # taps of the convolutions of q, k and v (attention, delta)
+    conv: int = 0                       # taps of the convolutions of q, k and v (attention, delta); 0: none
     scale: Optional[float] = None       # attention
     window: Optional[int] = None        # attention: mask.size
     pool: int = 0                       # attention: mask.pool
@@ -100,7 +100,7 @@ def _mixer(kind: str, mf: Fields, index: int, entries) -> SuripelMixer:
     kv_heads = mf.integer("kv_heads", default=heads)
     if heads % kv_heads:
         raise ConfigError(f"{mf.where}: heads = {heads} is no multiple of kv_heads = {kv_heads}")
-    conv = mf.integer("conv", default=1, hi=16)
+    conv = mf.integer("conv", default=0, hi=16)     # absent: the projections go on as they are, and no taps are stored
     if kind == "delta":
         return SuripelMixer(kind, heads, kv_heads, dim, vdim, conv=conv)
     mask = mf.mapping("mask")

@@ -68,7 +68,7 @@ extern "C" int xr_qkv_store(void* q_out, void* k_cache, void* v_cache, const flo
 // blocks starts[b] / P .. (starts[b] + n) / P - 1 are complete now.  One workgroup per
 // (new block, kv head, request); blocks that do not exist leave at once.
 template <typename T>
-__global__ __launch_bounds__(64) void k_pool_blocks(T* __restrict__ pk, T* __restrict__ pv, const T* __restrict__ kc,
+__global__ __launch_bounds__(256) void k_pool_blocks(T* __restrict__ pk, T* __restrict__ pv, const T* __restrict__ kc,
                                                     const T* __restrict__ vc, const int* __restrict__ starts,
                                                     const int* __restrict__ cu_q, const int* __restrict__ block_table,
                                                     int table_stride, const int* __restrict__ pool_table, int pool_stride,
@@ -81,21 +81,23 @@ __global__ __launch_bounds__(64) void k_pool_blocks(T* __restrict__ pk, T* __res
     const int ppage = pool_table[(size_t)b * pool_stride + (blk >> page_shift)];
     const int poff = blk & page_mask;
     const float inv = 1.0f / (float)P;
-    for (int d = threadIdx.x; d < D; d += 64) {
+    // channels of the key, then channels of the value, a thread each; positions in ascending order
+    for (int e = threadIdx.x; e < D + Dv; e += 256) {
         float acc = 0.f;
-        for (int j = 0; j < P; ++j) {
-            const int pos = blk * P + j;
-            acc += ld<T>(kc, (((size_t)bt[pos >> page_shift] * Hk + h) * page_size + (pos & page_mask)) * D + d);
+        if (e < D) {
+            for (int j = 0; j < P; ++j) {
+                const int pos = blk * P + j;
+                acc += ld<T>(kc, (((size_t)bt[pos >> page_shift] * Hk + h) * page_size + (pos & page_mask)) * D + e);
+            }
+            st<T>(pk, (((size_t)ppage * Hk + h) * page_size + poff) * D + e, acc * inv);
+        } else {
+            const int d = e - D;
+            for (int j = 0; j < P; ++j) {
+                const int pos = blk * P + j;
+                acc += ld<T>(vc, (((size_t)bt[pos >> page_shift] * Hk + h) * Dv + d) * page_size + (pos & page_mask));
+            }
+            st<T>(pv, (((size_t)ppage * Hk + h) * Dv + d) * page_size + poff, acc * inv);
         }
-        st<T>(pk, (((size_t)ppage * Hk + h) * page_size + poff) * D + d, acc * inv);
-    }
-    for (int d = threadIdx.x; d < Dv; d += 64) {
-        float acc = 0.f;
-        for (int j = 0; j < P; ++j) {
-            const int pos = blk * P + j;
-            acc += ld<T>(vc, (((size_t)bt[pos >> page_shift] * Hk + h) * Dv + d) * page_size + (pos & page_mask));
-        }
-        st<T>(pv, (((size_t)ppage * Hk + h) * Dv + d) * page_size + poff, acc * inv);
     }
 }
 
@@ -109,11 +111,11 @@ extern "C" int xr_pool_blocks(void* pk, void* pv, const void* k_cache, const voi
     if (B == 0 || max_new_blocks <= 0) return XR_OK;
     dim3 grid(max_new_blocks, Hk, B);
     if (dtype == XR_F32)
-        k_pool_blocks<float><<<grid, 64, 0, stream>>>((float*)pk, (float*)pv, (const float*)k_cache, (const float*)v_cache,
+        k_pool_blocks<float><<<grid, 256, 0, stream>>>((float*)pk, (float*)pv, (const float*)k_cache, (const float*)v_cache,
                                                       starts, cu_q, block_table, table_stride, pool_table, pool_stride, Hk,
                                                       D, Dv, P, shift, page_size - 1, page_size);
     else if (dtype == XR_BF16)
-        k_pool_blocks<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)pk, (bf16_t*)pv, (const bf16_t*)k_cache,
+        k_pool_blocks<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)pk, (bf16_t*)pv, (const bf16_t*)k_cache,
                                                        (const bf16_t*)v_cache, starts, cu_q, block_table, table_stride,
                                                        pool_table, pool_stride, Hk, D, Dv, P, shift, page_size - 1, page_size);
     else { xr_set_error("pool_blocks: bad dtype %d", dtype); return XR_BAD_ARG; }
@@ -135,42 +137,84 @@ struct PoolAttnArgs {
     int size, P;
 };
 
-template <typename T>
+// VEC (bfloat16, key size a multiple of 8, pages of at least 8): a key's channels are read eight at
+// a time, and the values, which lie position by position inside a page, eight positions of a
+// channel at a time; tiles then begin on multiples of 8 (keys below `lo` in the first tile count as
+// absent), so a group of eight never leaves its page.
+__device__ inline void unpack8(uint4 w, float* f) {
+    f[0] = __uint_as_float(w.x << 16); f[1] = __uint_as_float(w.x & 0xffff0000u);
+    f[2] = __uint_as_float(w.y << 16); f[3] = __uint_as_float(w.y & 0xffff0000u);
+    f[4] = __uint_as_float(w.z << 16); f[5] = __uint_as_float(w.z & 0xffff0000u);
+    f[6] = __uint_as_float(w.w << 16); f[7] = __uint_as_float(w.w & 0xffff0000u);
+}
+
+template <typename T, bool VEC>
 __device__ inline void attend_range(const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ bt, int lo,
                                     int hi, const float* qs, int kvh, const PoolAttnArgs& a, float& m, float& l,
                                     float* acc, int lane) {
-    for (int k0 = lo; k0 < hi; k0 += 64) {
+    for (int k0 = VEC ? (lo & ~7) : lo; k0 < hi; k0 += 64) {
         const int key = k0 + lane;
-        const bool valid = key < hi;
+        const bool valid = key >= lo && key < hi;
         float s = -INFINITY;
         if (valid) {
             const T* kr = kc + (((size_t)bt[key >> a.page_shift] * a.Hk + kvh) * a.page_size + (key & a.page_mask)) * a.D;
             float dot = 0.f;
-            for (int d = 0; d < a.D; ++d) dot = fmaf(qs[d], ld<T>(kr, d), dot);
+            if (VEC) {
+                for (int d = 0; d < a.D; d += 8) {
+                    float f[8];
+                    unpack8(*reinterpret_cast<const uint4*>(kr + d), f);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) dot = fmaf(qs[d + i], f[i], dot);
+                }
+            } else {
+                for (int d = 0; d < a.D; ++d) dot = fmaf(qs[d], ld<T>(kr, d), dot);
+            }
             s = dot * a.scale;
         }
         const float mn = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - mn) : 0.f;
-        const float corr = expf(m - mn);
+        const float corr = mn == -INFINITY ? 1.f : expf(m - mn);
         l = l * corr + wave_sum(p);
 #pragma unroll
         for (int dd = 0; dd < AP_MAX_D / 64; ++dd) acc[dd] *= corr;
         const int nk = hi - k0 < 64 ? hi - k0 : 64;
-        for (int j = 0; j < nk; ++j) {
-            const float pj = __shfl(p, j, 64);
-            const int kj = k0 + j;
-            const T* vb = vc + ((size_t)bt[kj >> a.page_shift] * a.Hk + kvh) * a.Dv * a.page_size + (kj & a.page_mask);
+        if (VEC) {
+            for (int j0 = 0; j0 < nk; j0 += 8) {
+                const int kj = k0 + j0;
+                if (kj + 7 < lo) continue;              // eight keys below the range: their page may be gone
+                float pj[8];
 #pragma unroll
-            for (int dd = 0; dd < AP_MAX_D / 64; ++dd) {
-                const int d = lane + 64 * dd;
-                if (d < a.Dv) acc[dd] = fmaf(pj, ld<T>(vb, (size_t)d * a.page_size), acc[dd]);
+                for (int i = 0; i < 8; ++i) pj[i] = __shfl(p, j0 + i, 64);
+                const T* vb = vc + ((size_t)bt[kj >> a.page_shift] * a.Hk + kvh) * a.Dv * a.page_size + (kj & a.page_mask);
+#pragma unroll
+                for (int dd = 0; dd < AP_MAX_D / 64; ++dd) {
+                    const int d = lane + 64 * dd;
+                    if (d < a.Dv) {
+                        float f[8];
+                        unpack8(*reinterpret_cast<const uint4*>(vb + (size_t)d * a.page_size), f);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            if (pj[i] > 0.f) acc[dd] = fmaf(pj[i], f[i], acc[dd]);     // (what lies past the range is never multiplied)
+                    }
+                }
+            }
+        } else {
+            for (int j = 0; j < nk; ++j) {
+                const float pj = __shfl(p, j, 64);
+                const int kj = k0 + j;
+                const T* vb = vc + ((size_t)bt[kj >> a.page_shift] * a.Hk + kvh) * a.Dv * a.page_size + (kj & a.page_mask);
+#pragma unroll
+                for (int dd = 0; dd < AP_MAX_D / 64; ++dd) {
+                    const int d = lane + 64 * dd;
+                    if (d < a.Dv) acc[dd] = fmaf(pj, ld<T>(vb, (size_t)d * a.page_size), acc[dd]);
+                }
             }
         }
         m = mn;
     }
 }
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(64) void k_attention_pooled(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kc,
                                                          const T* __restrict__ vc, const T* __restrict__ pk,
                                                          const T* __restrict__ pv, PoolAttnArgs a) {
@@ -189,8 +233,8 @@ __global__ __launch_bounds__(64) void k_attention_pooled(T* __restrict__ out, co
     // blocks b with b P + P - 1 <= pos - size, i.e. b < (pos - size + 1) / P
     const int n_blocks = (a.P > 0 && pos - a.size + 1 > 0) ? (pos - a.size + 1) / a.P : 0;
     if (n_blocks > 0)
-        attend_range<T>(pk, pv, a.pool_table + (size_t)req * a.pool_stride, 0, n_blocks, qs, kvh, a, m, l, acc, lane);
-    attend_range<T>(kc, vc, a.block_table + (size_t)req * a.table_stride, lo, pos + 1, qs, kvh, a, m, l, acc, lane);
+        attend_range<T, VEC>(pk, pv, a.pool_table + (size_t)req * a.pool_stride, 0, n_blocks, qs, kvh, a, m, l, acc, lane);
+    attend_range<T, VEC>(kc, vc, a.block_table + (size_t)req * a.table_stride, lo, pos + 1, qs, kvh, a, m, l, acc, lane);
     T* orow = out + ((size_t)t * a.H + h) * a.Dv;
 #pragma unroll
     for (int dd = 0; dd < AP_MAX_D / 64; ++dd) {
@@ -206,7 +250,7 @@ __global__ __launch_bounds__(64) void k_attention_pooled(T* __restrict__ out, co
 // log2 and the sum), so that their merge adds the two.  A record of `extras` names a block of 32
 // rows (row = token x heads-in-group + head) and its slot: request, row0, slot, q0, q_len, start.
 // One wave a row.
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void k_pool_partial(float* __restrict__ part_o, float* __restrict__ part_ml,
                                                       const T* __restrict__ q, const T* __restrict__ pk,
                                                       const T* __restrict__ pv, const int* __restrict__ extras,
@@ -232,7 +276,7 @@ __global__ __launch_bounds__(256) void k_pool_partial(float* __restrict__ part_o
 #pragma unroll
     for (int dd = 0; dd < AP_MAX_D / 64; ++dd) acc[dd] = 0.f;
     if (n_blocks > 0)
-        attend_range<T>(pk, pv, a.pool_table + (size_t)req * a.pool_stride, 0, n_blocks, qs[wave], kvh, a, m, l, acc, lane);
+        attend_range<T, VEC>(pk, pv, a.pool_table + (size_t)req * a.pool_stride, 0, n_blocks, qs[wave], kvh, a, m, l, acc, lane);
     const size_t at = ((size_t)slot * a.Hk + kvh) * 32 + r;
     const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
@@ -258,10 +302,13 @@ extern "C" int xr_attention_pool_partial(float* part_o, float* part_ml, const vo
     if (n_extras == 0) return XR_OK;
     PoolAttnArgs a{nullptr, nullptr, nullptr, pool_table, 0, pool_stride, H, Hk, D, Dv, shift, page_size - 1, page_size, scale, size, P};
     dim3 grid((unsigned)n_extras * 8, Hk);
+    const bool vec = dtype == XR_BF16 && D % 8 == 0 && page_size >= 8;
     if (dtype == XR_F32)
-        k_pool_partial<float><<<grid, 256, 0, stream>>>(part_o, part_ml, (const float*)q, (const float*)pk, (const float*)pv, extras, a);
+        k_pool_partial<float, false><<<grid, 256, 0, stream>>>(part_o, part_ml, (const float*)q, (const float*)pk, (const float*)pv, extras, a);
+    else if (dtype == XR_BF16 && vec)
+        k_pool_partial<bf16_t, true><<<grid, 256, 0, stream>>>(part_o, part_ml, (const bf16_t*)q, (const bf16_t*)pk, (const bf16_t*)pv, extras, a);
     else if (dtype == XR_BF16)
-        k_pool_partial<bf16_t><<<grid, 256, 0, stream>>>(part_o, part_ml, (const bf16_t*)q, (const bf16_t*)pk, (const bf16_t*)pv, extras, a);
+        k_pool_partial<bf16_t, false><<<grid, 256, 0, stream>>>(part_o, part_ml, (const bf16_t*)q, (const bf16_t*)pk, (const bf16_t*)pv, extras, a);
     else { xr_set_error("pooled partial: bad dtype %d", dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("attention_pool_partial");
     return XR_OK;
@@ -281,12 +328,16 @@ extern "C" int xr_attention_pooled(void* out, const void* q, const void* k_cache
     PoolAttnArgs a{positions, req_of_token, block_table, pool_table, table_stride, pool_stride, H, Hk, D, Dv, shift,
                    page_size - 1, page_size, scale, size, P};
     dim3 grid(T, H);
+    const bool vec = dtype == XR_BF16 && D % 8 == 0 && page_size >= 8;
     if (dtype == XR_F32)
-        k_attention_pooled<float><<<grid, 64, 0, stream>>>((float*)out, (const float*)q, (const float*)k_cache,
-                                                           (const float*)v_cache, (const float*)pk, (const float*)pv, a);
+        k_attention_pooled<float, false><<<grid, 64, 0, stream>>>((float*)out, (const float*)q, (const float*)k_cache,
+                                                                  (const float*)v_cache, (const float*)pk, (const float*)pv, a);
+    else if (dtype == XR_BF16 && vec)
+        k_attention_pooled<bf16_t, true><<<grid, 64, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
+                                                                  (const bf16_t*)v_cache, (const bf16_t*)pk, (const bf16_t*)pv, a);
     else if (dtype == XR_BF16)
-        k_attention_pooled<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
-                                                            (const bf16_t*)v_cache, (const bf16_t*)pk, (const bf16_t*)pv, a);
+        k_attention_pooled<bf16_t, false><<<grid, 64, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
+                                                                   (const bf16_t*)v_cache, (const bf16_t*)pk, (const bf16_t*)pv, a);
     else { xr_set_error("pooled attention: bad dtype %d", dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("attention_pooled");
     return XR_OK;

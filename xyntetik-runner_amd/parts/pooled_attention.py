@@ -44,9 +44,9 @@ class PooledWindowAttention(Mixer):
             raise ValueError(f"attention head sizes {self.head_dim}/{self.v_head_dim} are outside what the kernels take (1 to {MAX_HEAD_DIM})")
         self.window, self.pool = int(window), int(pool)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
-        self.conv_taps = int(conv_taps)
-        if not (1 <= self.conv_taps <= 16):
-            raise ValueError(f"attention: {conv_taps} convolution taps (1 to 16)")
+        self.conv_taps = int(conv_taps)      # 0: no convolution, and no tensors of one
+        if not (0 <= self.conv_taps <= 16):
+            raise ValueError(f"attention: {conv_taps} convolution taps (0 to 16)")
         need = max(self.window, self.pool)
         self.keep = max(int(keep), need) if keep is not None else need
         self.kv_shared = bool(kv_shared)
@@ -79,7 +79,8 @@ class PooledWindowAttention(Mixer):
         specs = {}
         for name, rows in self._projections():
             specs[name] = ParamSpec((rows, E))
-            specs[name + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal:0.6")
+            if self.conv_taps:
+                specs[name + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal:0.6")
         specs[self.names[3]] = ParamSpec((E, self.num_heads * self.v_head_dim))
         return specs
 
@@ -87,7 +88,8 @@ class PooledWindowAttention(Mixer):
         self.rt = rt
         mats = [tensors[name] for name, _ in self._projections()]
         self.w_in = rt.ops.pack_weight(torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0])
-        self.w_conv = torch.cat([tensors[name + self.conv_suffix].float() for name, _ in self._projections()], dim=0).contiguous()
+        self.w_conv = (torch.cat([tensors[name + self.conv_suffix].float() for name, _ in self._projections()], dim=0).contiguous()
+                       if self.conv_taps else None)
         self.w_out = rt.ops.pack_weight(tensors[self.names[3]])
 
     def _attend(self, ctx, cache, h):
@@ -98,7 +100,7 @@ class PooledWindowAttention(Mixer):
         if writes == self.kv_shared:
             raise ValueError("pooled attention: a layer stores its keys and values exactly when it projects them")
         proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
-        y = ops.causal_conv(proj, self.w_conv, cache.states.get("mixer.conv"), ctx, torch.float32)
+        y = ops.causal_conv(proj, self.w_conv, cache.states.get("mixer.conv"), ctx, torch.float32) if self.conv_taps else proj
         q = ops.qkv_store(y[:, :Q], y[:, Q:Q + K] if writes else None, y[:, Q + K:] if writes else None,
                           cache.k, cache.v, ctx, cache.group, H, G, D, Dv, cache.page_size, self.rt.dtype)
         if P and cache.pool_owns:

@@ -101,8 +101,8 @@ class GatedDelta(Mixer):
                  a_name: str = "a", a_log_name: str = "A_log", dt_bias_name: str = "dt_bias", norm_name: str = "norm",
                  g_name: str = "g", o_name: str = "o", conv_suffix: str = ".conv"):
         _check_sizes("gated delta rule", num_heads, num_kv_heads, head_dim, v_head_dim)
-        if not (1 <= int(conv_taps) <= 16):
-            raise ValueError(f"gated delta rule: {conv_taps} convolution taps (1 to 16)")
+        if not (0 <= int(conv_taps) <= 16):          # 0: no convolution (SiLU alone), and no tensors of one
+            raise ValueError(f"gated delta rule: {conv_taps} convolution taps (0 to 16)")
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.head_dim, self.v_head_dim = int(head_dim), int(v_head_dim)
         self.conv_taps, self.eps = int(conv_taps), float(eps)
@@ -124,7 +124,8 @@ class GatedDelta(Mixer):
         specs = {}
         for key, rows in (("q", self.qk_size), ("k", self.qk_size), ("v", self.v_size)):
             specs[n[key]] = ParamSpec((rows, E))
-            specs[n[key] + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal:0.6")
+            if self.conv_taps:
+                specs[n[key] + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal:0.6")
         specs[n["b"]] = ParamSpec((H, E))
         specs[n["a"]] = ParamSpec((H, E))
         specs[n["a_log"]] = ParamSpec((H,), role="vector", init="normal:0.5")
@@ -138,7 +139,10 @@ class GatedDelta(Mixer):
         self.rt = rt
         n = self.names
         self.w_in = rt.ops.pack_weight(torch.cat([tensors[n[key]] for key in ("q", "k", "v", "g", "b", "a")], dim=0).contiguous())
-        self.w_conv = torch.cat([tensors[n[key] + self.conv_suffix].float() for key in ("q", "k", "v")], dim=0).contiguous()
+        if self.conv_taps:
+            self.w_conv = torch.cat([tensors[n[key] + self.conv_suffix].float() for key in ("q", "k", "v")], dim=0).contiguous()
+        else:       # one tap of weight 1: the kernel's SiLU alone
+            self.w_conv = torch.ones((self.conv_size, 1), dtype=torch.float32, device=rt.device)
         self.a_log = tensors[n["a_log"]].float().contiguous()
         self.dt_bias = tensors[n["dt_bias"]].float().contiguous()
         self.w_norm = tensors[n["norm"]].float().contiguous()
