@@ -285,9 +285,9 @@ def measure_prefill_in_portions(runner, cfg, T, portion, seed):
 
 def suripel_config(width, layers, vocab=32000):
     """A Suripel model of real layer sizes: heads of 128, four query heads a key/value head, a
-    window of 1,024 with blocks of 64, every mixer in turn (the second attention of each six reads
-    the first one's keys and values), a dense feed-forward with as many weights as a gated one of
-    3.5 x width."""
+    window of 1,024 with blocks of 64, the mixers in turn (of every six layers: retention, attention,
+    delta, an attention that reads the first one's keys and values, retention, delta), a dense
+    feed-forward with as many weights as a gated one of 3.5 x width."""
     H = width // 128
     ff = {"kind": "dense", "ff": int(width * 5.25)}
 
@@ -298,12 +298,12 @@ def suripel_config(width, layers, vocab=32000):
             m["kv_from"] = kv_from
         return {"type": "attention", "mixer": m, "mlp": ff}
     delta = {"type": "delta", "mixer": {"heads": H, "kv_heads": max(1, H // 2), "dim": 128, "vdim": 128, "conv": 4}, "mlp": ff}
-    ret = {"type": "retention", "mixer": {"heads": H, "dim": 128, "vdim": 128, "decay": [1 - 2.0 ** (-5 - 5 * i / H) for i in range(H)],
+    ret = {"type": "retention", "mixer": {"heads": H, "dim": 128, "vdim": 128, "decay": [1 - 0.06 * 0.75 ** (8 * i / H) for i in range(H)],
                                           "rot": {"dims": 128, "base": 1e6}}, "mlp": ff}
     out = []
     for i in range(layers):
         k = i % 6
-        out.append(attn() if k == 0 else attn(kv_from=i - 4) if k == 4 else delta if k in (1, 5) else ret)
+        out.append(attn() if k == 1 else attn(kv_from=i - 2) if k == 3 else delta if k in (2, 5) else ret)
     return {"architecture": "Suripel", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "layers": out}
 
 

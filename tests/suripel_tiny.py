@@ -75,7 +75,7 @@ TINY_S3 = {
     "architecture": "Suripel", "vocab": 256, "width": 64, "norm": {"eps": 1e-5}, "canon": {"taps": 4},
     "layers": [
         with_ff(attention(4, 2, 32, 32, 40, 16, 4, 0.18), 96),
-        with_ff(retention(2, 32, 16, [0.96875, 0.998], rot=(32, 1e6)), 96),
+        with_ff(retention(2, 32, 16, [0.95, 0.998], rot=(32, 250000.0)), 96),
         with_ff(attention(4, 2, 32, 32, 24, 8, 3, 0.18, kv_from=0), 96),
         with_ff(delta(2, 2, 32, 64, 4), 96),
         with_ff(attention(2, 1, 16, 48, 70, 32, 2, 0.25), 96),

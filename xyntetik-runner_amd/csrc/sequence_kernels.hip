@@ -99,44 +99,49 @@ __global__ __launch_bounds__(256) void k_causal_conv(TO* __restrict__ out, const
     st<TO>(out, (size_t)t * ld_out + c, acc);
 }
 
-// 32-bit rows whose width and strides are multiples of 4: a thread takes four channels, its loads
-// are 16 bytes (at 2,048 rows of 2,048 channels 26 us with a channel a thread).
-template <typename TO> __device__ inline void store4(TO* p, size_t i, float a, float b, float c, float d);
-template <> __device__ inline void store4<float>(float* p, size_t i, float a, float b, float c, float d) {
-    *reinterpret_cast<float4*>(p + i) = make_float4(a, b, c, d);
-}
-template <> __device__ inline void store4<bf16_t>(bf16_t* p, size_t i, float a, float b, float c, float d) {
-    *reinterpret_cast<uint2*>(p + i) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
-}
-
-template <typename TO>
-__global__ __launch_bounds__(256) void k_causal_conv4(TO* __restrict__ out, const float* __restrict__ u,
-                                                      const float* __restrict__ w, const float* __restrict__ state,
-                                                      const int* __restrict__ cu_q, const int* __restrict__ slots,
-                                                      const int* __restrict__ req_of_token, int C, int taps, int ld_u,
-                                                      int ld_out, int residual, int act) {
-    const int t = blockIdx.y;
-    const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
+// Many rows: a thread takes CONV_ROWS consecutive rows of its channel.  What a row needs before its
+// first input (its request, the request's first row and state row) are three loads that wait for
+// each other; with a row a thread a workgroup spent most of its life on them (2,048 rows of 2,048
+// channels: 26 us), here the rows' chains run side by side.  (Four channels a thread with 16-byte
+// loads was slower still: 34 us.)
+#define CONV_ROWS 8
+template <typename TU, typename TO>
+__global__ __launch_bounds__(256) void k_causal_conv_rows(TO* __restrict__ out, const TU* __restrict__ u,
+                                                          const float* __restrict__ w, const TU* __restrict__ state,
+                                                          const int* __restrict__ cu_q, const int* __restrict__ slots,
+                                                          const int* __restrict__ req_of_token, int T, int C, int taps,
+                                                          int ld_u, int ld_out, int residual, int act) {
+    const int t0 = blockIdx.y * CONV_ROWS;
+    const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
-    const int b = req_of_token[t];
-    const int row0 = cu_q[b];
-    const int i = t - row0;
-    const float* srow = state + (size_t)slots[b] * (taps - 1) * C;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f), val = acc;
-    for (int j = 0; j < taps; ++j) {
-        const int s = i - (taps - 1) + j;
-        val = *reinterpret_cast<const float4*>(s >= 0 ? u + (size_t)(row0 + s) * ld_u + c : srow + (size_t)(taps - 1 + s) * C + c);
-        acc.x = fmaf(w[(size_t)c * taps + j], val.x, acc.x);
-        acc.y = fmaf(w[(size_t)(c + 1) * taps + j], val.y, acc.y);
-        acc.z = fmaf(w[(size_t)(c + 2) * taps + j], val.z, acc.z);
-        acc.w = fmaf(w[(size_t)(c + 3) * taps + j], val.w, acc.w);
+    int row0[CONV_ROWS], slot[CONV_ROWS];
+#pragma unroll
+    for (int r = 0; r < CONV_ROWS; ++r) {
+        const int b = req_of_token[t0 + r < T ? t0 + r : T - 1];
+        row0[r] = cu_q[b];
+        slot[r] = slots[b];
     }
-    if (residual) { acc.x += val.x; acc.y += val.y; acc.z += val.z; acc.w += val.w; }     // (the last tap's input is the row itself)
-    if (act == XR_CONV_SILU) {
-        acc.x = acc.x / (1.0f + expf(-acc.x)); acc.y = acc.y / (1.0f + expf(-acc.y));
-        acc.z = acc.z / (1.0f + expf(-acc.z)); acc.w = acc.w / (1.0f + expf(-acc.w));
+    float wt[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) wt[j] = j < taps ? w[(size_t)c * taps + j] : 0.f;
+#pragma unroll
+    for (int r = 0; r < CONV_ROWS; ++r) {
+        const int t = t0 + r;
+        if (t >= T) break;
+        const int i = t - row0[r];
+        const TU* srow = state + (size_t)slot[r] * (taps - 1) * C;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+            if (j >= taps) break;
+            const int s = i - (taps - 1) + j;
+            const float val = s >= 0 ? ld<TU>(u, (size_t)(row0[r] + s) * ld_u + c) : ld<TU>(srow, (size_t)(taps - 1 + s) * C + c);
+            acc = fmaf(wt[j], val, acc);
+        }
+        if (residual) acc += ld<TU>(u, (size_t)t * ld_u + c);
+        if (act == XR_CONV_SILU) acc = acc / (1.0f + expf(-acc));
+        st<TO>(out, (size_t)t * ld_out + c, acc);
     }
-    store4<TO>(out, (size_t)t * ld_out + c, acc.x, acc.y, acc.z, acc.w);
 }
 
 template <typename TU>
@@ -176,28 +181,18 @@ extern "C" int xr_causal_conv(void* out, const void* u, const float* w, void* st
     if (T == 0 || B == 0) return XR_OK;
     const int fuse = one_row_each && taps > 1 ? 1 : 0;
     dim3 grid((C + 255) / 256, T), sgrid((C + 255) / 256, B);
+    dim3 rgrid((C + 255) / 256, (T + CONV_ROWS - 1) / CONV_ROWS);
 #define CC(TU, TO)                                                                                                   \
     do {                                                                                                             \
+        if (T >= 8 * CONV_ROWS && !fuse)                                                                             \
+            k_causal_conv_rows<TU, TO><<<rgrid, 256, 0, stream>>>((TO*)out, (const TU*)u, w, (const TU*)state, cu_q,  \
+                                                                  slots, req_of_token, T, C, taps, ld_u, ld_out,     \
+                                                                  residual, act);                                    \
+        else                                                                                                         \
         k_causal_conv<TU, TO><<<grid, 256, 0, stream>>>((TO*)out, (const TU*)u, w, (TU*)state, cu_q, slots,           \
                                                         req_of_token, C, taps, ld_u, ld_out, residual, act, fuse);    \
         if (taps > 1 && !fuse) k_conv_state<TU><<<sgrid, 256, 0, stream>>>((TU*)state, (const TU*)u, cu_q, slots, C, taps, ld_u); \
     } while (0)
-    // many rows of 32-bit inputs: four channels a thread (the state is then rewritten by its own kernel)
-    const bool wide = !fuse && T >= 64 && u_dtype == XR_F32 && C % 4 == 0 && ld_u % 4 == 0 && ld_out % 4 == 0 &&
-                      ((uintptr_t)u % 16) == 0 && ((uintptr_t)out % 16) == 0 && (state == nullptr || ((uintptr_t)state % 16) == 0);
-    if (wide) {
-        dim3 grid4((C / 4 + 255) / 256, T);
-        if (out_dtype == XR_F32)
-            k_causal_conv4<float><<<grid4, 256, 0, stream>>>((float*)out, (const float*)u, w, (const float*)state, cu_q, slots,
-                                                             req_of_token, C, taps, ld_u, ld_out, residual, act);
-        else if (out_dtype == XR_BF16)
-            k_causal_conv4<bf16_t><<<grid4, 256, 0, stream>>>((bf16_t*)out, (const float*)u, w, (const float*)state, cu_q, slots,
-                                                              req_of_token, C, taps, ld_u, ld_out, residual, act);
-        else { xr_set_error("causal_conv: bad dtypes %d %d", u_dtype, out_dtype); return XR_BAD_ARG; }
-        if (taps > 1) k_conv_state<float><<<sgrid, 256, 0, stream>>>((float*)state, (const float*)u, cu_q, slots, C, taps, ld_u);
-        XR_CHECK_LAUNCH("causal_conv");
-        return XR_OK;
-    }
     if (u_dtype == XR_F32 && out_dtype == XR_F32) CC(float, float);
     else if (u_dtype == XR_F32 && out_dtype == XR_BF16) CC(float, bf16_t);
     else if (u_dtype == XR_BF16 && out_dtype == XR_BF16) CC(bf16_t, bf16_t);
