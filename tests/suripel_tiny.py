@@ -83,7 +83,19 @@ TINY_S3 = {
     ],
 }
 
-CONFIGS = {"S1": (TINY_S1, 11), "S2": (TINY_S2, 12), "S3": (TINY_S3, 13)}
+# no attention at all (no cache group, state only), a width that is no multiple of 8, one layer
+TINY_S4 = {
+    "architecture": "Suripel", "vocab": 61, "width": 50, "norm": {"eps": 1e-5}, "canon": {"taps": 1},
+    "layers": [with_ff(retention(1, 40, 72, [0.9], rot=(2, 100.0)), 30), with_ff(delta(1, 1, 36, 3, 5), None)],
+}
+
+# attention alone: one layer, one head, a window of one with blocks of two
+TINY_S5 = {
+    "architecture": "Suripel", "vocab": 80, "width": 32, "norm": {"eps": 1e-3}, "canon": {"taps": 5},
+    "layers": [with_ff(attention(1, 1, 16, 16, 1, 2, 2, 1.0), 48)],
+}
+
+CONFIGS = {"S1": (TINY_S1, 11), "S2": (TINY_S2, 12), "S3": (TINY_S3, 13), "S4": (TINY_S4, 14), "S5": (TINY_S5, 15)}
 
 
 def make_model(which: str, folder: str, std: float = 0.12) -> str:

@@ -30,6 +30,8 @@ WORKLOAD = {
     "S1": ([1, 4, 23, 64, 150], 20),        # 1 and 4: shorter than the taps; 64: ends on a page of 64, 16 and 8
     "S2": ([2, 9, 31, 100], 26),
     "S3": ([3, 70, 129, 330], 40),          # past several blocks, windows and pages of 64
+    "S4": ([2, 45], 12),
+    "S5": ([1, 37, 70], 10),
 }
 
 
@@ -90,7 +92,7 @@ def steps_for(schedule, reqs, plens, extra):
         return traces.tail_one_by_one(reqs, tail=extra)
     if schedule == "portions":
         return traces.portions(reqs)
-    return traces.mixed(reqs, plens, max_live=3, seed=5)
+    return traces.mixed(reqs, plens, max_live=min(3, len(reqs)), seed=5)
 
 
 @pytest.mark.parametrize("schedule", SCHEDULES)
@@ -103,6 +105,18 @@ def test_every_way_of_cutting_gives_the_plain_logits(models, tmp_path, which, pa
     check(traces.collect(steps, out, cfg["vocab"]), want, dtype, f"{which} {schedule}")
     if schedule == "tail":
         assert runner.graphs.replays > 0, "single tokens went through no recorded step"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which,page_size", [("S4", 16), ("S5", 16), ("S5", 64)])
+def test_models_of_one_kind_of_mixer(models, tmp_path, which, page_size, dtype):
+    """A model without attention has no cache group at all; one with attention alone no recurrent state."""
+    d, cfg, w, reqs, plens, want = models[which]
+    for schedule in ("tail", "mixed"):
+        steps = steps_for(schedule, reqs, plens, WORKLOAD[which][1])
+        out, runner = run_replay(d, dtype, steps, tmp_path / schedule, page_size, max_requests=3)
+        assert (len(runner.manager.groups) == 0) == (which == "S4")
+        check(traces.collect(steps, out, cfg["vocab"]), want, dtype, f"{which} {schedule}")
 
 
 def test_mixed_batch_equals_each_request_alone_bit_for_bit_in_kind(models, tmp_path):
