@@ -105,6 +105,10 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
         }
     };
     fetch(0);
+    float4 qp[DPER / 4];            // (delta rule) the query of the token before, whose read-out is still owed
+#pragma unroll
+    for (int j = 0; j < DPER / 4; ++j) qp[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    int prev_row = -1;
     for (int c0 = 0; c0 < n; c0 += REC_TOKENS) {
         const int nt = n - c0 < REC_TOKENS ? n - c0 : REC_TOKENS;
         __syncthreads();
@@ -117,43 +121,90 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
         if (MODE == XR_REC_DELTA && tid < REC_TOKENS) { bs[tid] = rb; gs[tid] = rg; }
         __syncthreads();
         if (c0 + REC_TOKENS < n) fetch(c0 + REC_TOKENS);
-        for (int tt = 0; tt < nt; ++tt) {
-            const float4* kq = &ks[tt][r * (DPER / 4)];
-            const float4* qq = &qs[tt][r * (DPER / 4)];
-            const float vv = vs[tt][cl];
-            float4 kk[DPER / 4], q4[DPER / 4];
-#pragma unroll
-            for (int j = 0; j < DPER / 4; ++j) { kk[j] = kq[j]; q4[j] = qq[j]; }
-            float o0 = 0.f, o1 = 0.f;
-            if (MODE == XR_REC_DELTA) {
-                const float g = gs[tt];
-                float d0 = 0.f, d1 = 0.f;        // two chains of sums, added at the end
+        if (MODE == XR_REC_DELTA) {
+            // The state's chain a token is: sum over the column (S . k), u, one multiply-add.  The
+            // read-out (S . q) is off that chain but a wave issues in order, so the read-out of the
+            // token before runs in the same pass over S as this token's sum: two chains side by side.
+            for (int tt = 0; tt < nt; ++tt) {
+                const float4* kq = &ks[tt][r * (DPER / 4)];
+                const float4* qq = &qs[tt][r * (DPER / 4)];
+                const float vv = vs[tt][cl], g = gs[tt], bt = bs[tt];
+                float4 kk[DPER / 4];
+                float d0 = 0.f, d1 = 0.f, p0 = 0.f, p1 = 0.f;
 #pragma unroll
                 for (int j = 0; j < DPER; j += 4) {
-                    S[j] *= g; S[j + 1] *= g; S[j + 2] *= g; S[j + 3] *= g;
+                    kk[j >> 2] = kq[j >> 2];
                     d0 = fmaf(S[j], kk[j >> 2].x, d0); d1 = fmaf(S[j + 1], kk[j >> 2].y, d1);
                     d0 = fmaf(S[j + 2], kk[j >> 2].z, d0); d1 = fmaf(S[j + 3], kk[j >> 2].w, d1);
+                    p0 = fmaf(S[j], qp[j >> 2].x, p0); p1 = fmaf(S[j + 1], qp[j >> 2].y, p1);
+                    p0 = fmaf(S[j + 2], qp[j >> 2].z, p0); p1 = fmaf(S[j + 3], qp[j >> 2].w, p1);
                 }
-                const float u = bs[tt] * (vv - group_sum<R>(d0 + d1));
+                const float dsum = group_sum<R>(d0 + d1), psum = group_sum<R>(p0 + p1);
+                if (prev_row >= 0 && live && r == 0) a.out[((size_t)prev_row * a.H + h) * a.Dv + col] = psum;
+                const float u = bt * (vv - g * dsum);          // S^T k of the decayed state = g (S^T k)
 #pragma unroll
                 for (int j = 0; j < DPER; j += 4) {
-                    S[j] = fmaf(kk[j >> 2].x, u, S[j]); S[j + 1] = fmaf(kk[j >> 2].y, u, S[j + 1]);
-                    S[j + 2] = fmaf(kk[j >> 2].z, u, S[j + 2]); S[j + 3] = fmaf(kk[j >> 2].w, u, S[j + 3]);
-                    o0 = fmaf(S[j], q4[j >> 2].x, o0); o1 = fmaf(S[j + 1], q4[j >> 2].y, o1);
-                    o0 = fmaf(S[j + 2], q4[j >> 2].z, o0); o1 = fmaf(S[j + 3], q4[j >> 2].w, o1);
+                    S[j] = fmaf(g, S[j], kk[j >> 2].x * u); S[j + 1] = fmaf(g, S[j + 1], kk[j >> 2].y * u);
+                    S[j + 2] = fmaf(g, S[j + 2], kk[j >> 2].z * u); S[j + 3] = fmaf(g, S[j + 3], kk[j >> 2].w * u);
+                    qp[j >> 2] = qq[j >> 2];
                 }
-            } else {
+                prev_row = row0 + c0 + tt;
+            }
+        } else {
+            // Retention's chain is one multiply-add a token; four tokens' read-outs run side by side.
+            int tt = 0;
+            for (; tt + 4 <= nt; tt += 4) {
+                float oo[4];
 #pragma unroll
-                for (int j = 0; j < DPER; j += 4) {
-                    S[j] = fmaf(dec, S[j], kk[j >> 2].x * vv); S[j + 1] = fmaf(dec, S[j + 1], kk[j >> 2].y * vv);
-                    S[j + 2] = fmaf(dec, S[j + 2], kk[j >> 2].z * vv); S[j + 3] = fmaf(dec, S[j + 3], kk[j >> 2].w * vv);
-                    o0 = fmaf(S[j], q4[j >> 2].x, o0); o1 = fmaf(S[j + 1], q4[j >> 2].y, o1);
-                    o0 = fmaf(S[j + 2], q4[j >> 2].z, o0); o1 = fmaf(S[j + 3], q4[j >> 2].w, o1);
+                for (int x = 0; x < 4; ++x) {
+                    const float4* kq = &ks[tt + x][r * (DPER / 4)];
+                    const float4* qq = &qs[tt + x][r * (DPER / 4)];
+                    const float vv = vs[tt + x][cl];
+                    float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+                    for (int j = 0; j < DPER; j += 4) {
+                        const float4 kk = kq[j >> 2], q4 = qq[j >> 2];
+                        S[j] = fmaf(dec, S[j], kk.x * vv); S[j + 1] = fmaf(dec, S[j + 1], kk.y * vv);
+                        S[j + 2] = fmaf(dec, S[j + 2], kk.z * vv); S[j + 3] = fmaf(dec, S[j + 3], kk.w * vv);
+                        o0 = fmaf(S[j], q4.x, o0); o1 = fmaf(S[j + 1], q4.y, o1);
+                        o0 = fmaf(S[j + 2], q4.z, o0); o1 = fmaf(S[j + 3], q4.w, o1);
+                    }
+                    oo[x] = o0 + o1;
+                }
+#pragma unroll
+                for (int x = 0; x < 4; ++x) oo[x] = group_sum<R>(oo[x]);
+                if (live && r == 0) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) a.out[((size_t)(row0 + c0 + tt + x) * a.H + h) * a.Dv + col] = oo[x];
                 }
             }
-            const float o = group_sum<R>(o0 + o1);
-            if (live && r == 0) a.out[((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col] = o;
+            for (; tt < nt; ++tt) {
+                const float4* kq = &ks[tt][r * (DPER / 4)];
+                const float4* qq = &qs[tt][r * (DPER / 4)];
+                const float vv = vs[tt][cl];
+                float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+                for (int j = 0; j < DPER; j += 4) {
+                    const float4 kk = kq[j >> 2], q4 = qq[j >> 2];
+                    S[j] = fmaf(dec, S[j], kk.x * vv); S[j + 1] = fmaf(dec, S[j + 1], kk.y * vv);
+                    S[j + 2] = fmaf(dec, S[j + 2], kk.z * vv); S[j + 3] = fmaf(dec, S[j + 3], kk.w * vv);
+                    o0 = fmaf(S[j], q4.x, o0); o1 = fmaf(S[j + 1], q4.y, o1);
+                    o0 = fmaf(S[j + 2], q4.z, o0); o1 = fmaf(S[j + 3], q4.w, o1);
+                }
+                const float o = group_sum<R>(o0 + o1);
+                if (live && r == 0) a.out[((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col] = o;
+            }
         }
+    }
+    if (MODE == XR_REC_DELTA) {      // the last token's read-out
+        float p0 = 0.f, p1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < DPER; j += 4) {
+            p0 = fmaf(S[j], qp[j >> 2].x, p0); p1 = fmaf(S[j + 1], qp[j >> 2].y, p1);
+            p0 = fmaf(S[j + 2], qp[j >> 2].z, p0); p1 = fmaf(S[j + 3], qp[j >> 2].w, p1);
+        }
+        const float psum = group_sum<R>(p0 + p1);
+        if (prev_row >= 0 && live && r == 0) a.out[((size_t)prev_row * a.H + h) * a.Dv + col] = psum;
     }
     if (live) {
 #pragma unroll
