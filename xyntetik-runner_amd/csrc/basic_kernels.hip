@@ -384,6 +384,31 @@ extern "C" int xr_fill_rows(void* base, const int* rows, int n_rows, size_t row_
     return XR_OK;
 }
 
+// The same for many arrays at once (every state tensor of every layer when a request begins): array a
+// has rows of row_words[a] words at bases[a]; one launch instead of one an array.
+__global__ void k_fill_rows_many(uint32_t* const* __restrict__ bases, const size_t* __restrict__ row_words,
+                                 const int* __restrict__ rows, uint32_t value) {
+    const size_t words = row_words[blockIdx.z];
+    const int r = rows[blockIdx.y];
+    if (r < 0) return;
+    uint32_t* row = bases[blockIdx.z] + (size_t)r * words;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (size_t)gridDim.x * blockDim.x) row[i] = value;
+}
+
+// bases, row_words: device arrays of n_arrays entries; rows: n_rows row numbers on the device.
+extern "C" int xr_fill_rows_many(void* const* bases, const size_t* row_words, int n_arrays, size_t max_row_words,
+                                 const int* rows, int n_rows, uint32_t value, hipStream_t stream) {
+    if (n_arrays <= 0 || n_rows <= 0 || max_row_words == 0) return XR_OK;
+    XR_REQUIRE(bases && row_words && rows, "fill_rows_many: an operand is missing");
+    XR_REQUIRE(n_arrays <= 65535 && n_rows <= 65535, "fill_rows_many: %d arrays, %d rows (at most 65535 each)", n_arrays, n_rows);
+    size_t blocks = (max_row_words + 255) / 256;
+    if (blocks > 64) blocks = 64;           // longer rows: a block strides over its row
+    dim3 grid((unsigned)blocks, n_rows, n_arrays);
+    k_fill_rows_many<<<grid, 256, 0, stream>>>((uint32_t* const*)bases, row_words, rows, value);
+    XR_CHECK_LAUNCH("fill_rows_many");
+    return XR_OK;
+}
+
 // ---------------------------------------------------------------- dtype conversion
 template <typename TI, typename TO>
 __global__ void k_convert(TO* __restrict__ out, const TI* __restrict__ in, size_t n) {

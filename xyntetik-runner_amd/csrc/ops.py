@@ -49,6 +49,7 @@ _PROTOS = {
     "xr_gate_mul": [_p, _p, _i, _i, _i, _i, _i, _p],
     "xr_add": [_p, _p, _sz, _i, _p],
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
+    "xr_fill_rows_many": [_p, _p, _i, _sz, _p, _i, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_stream_read": [_p, _sz, _p, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
@@ -262,6 +263,29 @@ class Ops:
             raise KernelError("fill_rows_: a row must be a multiple of 4 bytes")
         self.lib.check(self.lib.xr_fill_rows(base.data_ptr(), _ptr(rows), int(n_rows), row_bytes // 4,
                                              value_bits & 0xFFFFFFFF, _stream()))
+
+    def row_filler(self, arrays):
+        """A callable ``fill(rows, n_rows, value_bits=0)`` that sets the rows ``rows`` (device int32) of
+        every array of ``arrays`` (first axis) to a 32-bit pattern in one launch; None if there are none."""
+        arrays = list(arrays)
+        if not arrays:
+            return None
+        self._dev(*arrays)
+        words = []
+        for t in arrays:
+            self._contig(t, "row_filler array")
+            row_bytes = t[0].numel() * t.element_size()
+            if row_bytes % 4:
+                raise KernelError("row_filler: a row must be a multiple of 4 bytes")
+            words.append(row_bytes // 4)
+        device = arrays[0].device
+        bases = torch.tensor([t.data_ptr() for t in arrays], dtype=torch.int64, device=device)
+        sizes = torch.tensor(words, dtype=torch.int64, device=device)
+
+        def fill(rows: torch.Tensor, n_rows: int, value_bits: int = 0, _keep=(arrays, bases, sizes)) -> None:
+            self.lib.check(self.lib.xr_fill_rows_many(bases.data_ptr(), sizes.data_ptr(), len(arrays), max(words),
+                                                      rows.data_ptr(), int(n_rows), value_bits & 0xFFFFFFFF, _stream()))
+        return fill
 
     def convert(self, x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
         self._dev(x)

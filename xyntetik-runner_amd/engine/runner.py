@@ -200,9 +200,7 @@ class ModelRunner:
         """The state rows of requests that use their slot for the first time begin at zero."""
         if not slots:
             return
-        rows = None
-        for lc in self.storage.layers:
-            for state in lc.states.values():
-                if rows is None:
-                    rows = torch.tensor(slots, dtype=torch.int32, device=self.device)
-                self.ops.fill_rows_(state, rows, len(slots), 0)
+        if not hasattr(self, "_fill_states"):       # every state tensor of every layer, in one launch
+            self._fill_states = self.ops.row_filler(st for lc in self.storage.layers for st in lc.states.values())
+        if self._fill_states is not None:
+            self._fill_states(torch.tensor(slots, dtype=torch.int32, device=self.device), len(slots), 0)
