@@ -250,6 +250,25 @@ def test_retention(ops, H, D, Dv):
         close(got[b], want[b], 5e-6, f"retention request {b}")
 
 
+@pytest.mark.parametrize("H,D,Dv", [(2, 64, 48), (1, 20, 70)])
+def test_retention_in_chunks_side_by_side(ops, H, D, Dv):
+    """A portion long enough to be cut into chunks that run side by side (1,300 rows: five chunks and a
+    rest), in one step with a short request and one that ends on a chunk's edge; then the state each
+    left is carried on token by token."""
+    rng = np.random.default_rng(D)
+    lens = [1300 + 9, 40 + 9, 1024 + 9]
+    qs = [rng.normal(size=(n, H, D)) for n in lens]
+    ks = [rng.normal(size=(n, H, D)) * D ** -0.5 for n in lens]
+    vs = [rng.normal(size=(n, H, Dv)) for n in lens]
+    decay = [0.97, 0.9995][:H]
+    want = [S.retention(q, k, v, decay) for q, k, v in zip(qs, ks, vs)]
+    assert max(lens) - 9 >= ops.RETENTION_CHUNKED_FROM
+    plans = [[(0, n - 9)] + [(i, 1) for i in range(n - 9, n)] for n in lens]
+    got = run_recurrence(ops, "retention", qs, ks, vs, decay, H, H, D, Dv, plans, [2, 0, 1], 3)
+    for b in range(3):
+        close(got[b], want[b], 2e-5, f"chunked retention request {b}")
+
+
 def test_delta_prepare(ops):
     rng = np.random.default_rng(3)
     T, G, H, D = 5, 2, 4, 12

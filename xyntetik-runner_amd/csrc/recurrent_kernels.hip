@@ -35,6 +35,17 @@ struct RecArgs {
     const int* cu_q;
     const int* slots;
     int H, G, D, Dv, ld, ld_g;   // row strides of q/k/v and of beta/gate
+    // Retention over a long portion, cut into chunks of chunk_len rows that run side by side (its decay is
+    // one number a head, so S_t = (the chunk's own sum from zero) + decay^(i+1) x (the state before the
+    // chunk), i the row's place in the chunk):
+    //   pass 1: every chunk runs the recurrence from zero (the first from the request's state), writes its
+    //           read-outs and leaves its last state in scratch [request x chunk][head][J][Dv][R];
+    //   k_retention_carry turns those into every chunk's true first state, and the request's new state;
+    //   pass 2: every chunk but the first runs again from its true first state with nothing written
+    //           (v = 0: the state just decays) and adds its read-outs to those of pass 1.
+    // pass 0: one workgroup runs the whole portion.
+    int pass, chunk_len, n_chunks;
+    float* scratch;
 };
 
 // the value of lane (l ^ 1), (l ^ 2) of a quad, or of the lane 4 / 8 further round a row of 16
@@ -58,18 +69,28 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
     __shared__ float4 ks[REC_TOKENS][R * DPER / 4];
     __shared__ float vs[REC_TOKENS][COLS];
     __shared__ float bs[REC_TOKENS], gs[REC_TOKENS];
-    const int b = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
+    const int h = blockIdx.y, tid = threadIdx.x;
     const int cl = tid / R, r = tid % R;
     const int col = blockIdx.x * COLS + cl;
     const bool live = col < a.Dv;
-    const int row0 = a.cu_q[b], n = a.cu_q[b + 1] - row0;
+    const int pass = MODE == XR_REC_RETENTION ? a.pass : 0;
+    int b = blockIdx.z, chunk = 0;
+    if (pass) { chunk = b % a.n_chunks; b /= a.n_chunks; }
+    int row0 = a.cu_q[b], n = a.cu_q[b + 1] - row0;
+    if (pass) {
+        if (chunk * a.chunk_len >= n || (pass == 2 && chunk == 0)) return;
+        row0 += chunk * a.chunk_len;
+        n = n - chunk * a.chunk_len < a.chunk_len ? n - chunk * a.chunk_len : a.chunk_len;
+    }
     if (n <= 0) return;
     const int kvh = h / (a.H / a.G);
     const int J = (a.D + R - 1) / R;
     float* sp = a.state + (((size_t)a.slots[b] * a.H + h) * J) * a.Dv * R;
+    float* cp = pass ? a.scratch + ((((size_t)b * a.n_chunks + chunk) * a.H + h) * J) * a.Dv * R : nullptr;
+    const float* from = pass == 2 ? cp : (pass == 1 && chunk > 0) ? nullptr : sp;
     float S[DPER];
 #pragma unroll
-    for (int j = 0; j < DPER; ++j) S[j] = (live && j < J) ? sp[((size_t)j * a.Dv + col) * R + r] : 0.f;
+    for (int j = 0; j < DPER; ++j) S[j] = (live && j < J && from) ? from[((size_t)j * a.Dv + col) * R + r] : 0.f;
     const float dec = MODE == XR_REC_RETENTION ? a.decay[h] : 1.f;
     float* qf = reinterpret_cast<float*>(&qs[0][0]);
     float* kf = reinterpret_cast<float*>(&ks[0][0]);
@@ -96,7 +117,7 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
             const int idx = tid + i * 256;
             const int tt = idx / COLS, c = idx - tt * COLS;
             const int cc = blockIdx.x * COLS + c;
-            const bool ok = idx < REC_TOKENS * COLS && tt < nt && cc < a.Dv;
+            const bool ok = idx < REC_TOKENS * COLS && tt < nt && cc < a.Dv && pass != 2;
             rv[i] = ok ? a.v[(size_t)(row0 + c0 + tt) * a.ld + (size_t)h * a.Dv + cc] : 0.f;
         }
         if (MODE == XR_REC_DELTA && tid < nt) {
@@ -175,7 +196,10 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
                 for (int x = 0; x < 4; ++x) oo[x] = group_sum<R>(oo[x]);
                 if (live && r == 0) {
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) a.out[((size_t)(row0 + c0 + tt + x) * a.H + h) * a.Dv + col] = oo[x];
+                    for (int x = 0; x < 4; ++x) {
+                        float* dst = a.out + ((size_t)(row0 + c0 + tt + x) * a.H + h) * a.Dv + col;
+                        *dst = pass == 2 ? *dst + oo[x] : oo[x];
+                    }
                 }
             }
             for (; tt < nt; ++tt) {
@@ -192,7 +216,10 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
                     o0 = fmaf(S[j + 2], q4.z, o0); o1 = fmaf(S[j + 3], q4.w, o1);
                 }
                 const float o = group_sum<R>(o0 + o1);
-                if (live && r == 0) a.out[((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col] = o;
+                if (live && r == 0) {
+                    float* dst = a.out + ((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col;
+                    *dst = pass == 2 ? *dst + o : o;
+                }
             }
         }
     }
@@ -206,11 +233,35 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
         const float psum = group_sum<R>(p0 + p1);
         if (prev_row >= 0 && live && r == 0) a.out[((size_t)prev_row * a.H + h) * a.Dv + col] = psum;
     }
-    if (live) {
+    if (live && pass != 2) {
+        float* to = pass == 1 ? cp : sp;
 #pragma unroll
         for (int j = 0; j < DPER; ++j)
-            if (j < J) sp[((size_t)j * a.Dv + col) * R + r] = S[j];
+            if (j < J) to[((size_t)j * a.Dv + col) * R + r] = S[j];
     }
+}
+
+// Between the two passes over the chunks: scratch[b][c] holds chunk c's last state as if it had begun at
+// zero (chunk 0's is true).  In place, chunk by chunk: the true first state of chunk c (for pass 2), and
+// at the end the request's new state.  One thread an element of a head's state.
+__global__ __launch_bounds__(256) void k_retention_carry(RecArgs a, int per_head) {
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= per_head) return;
+    const int n = a.cu_q[b + 1] - a.cu_q[b];
+    if (n <= 0) return;
+    const int nc = (n + a.chunk_len - 1) / a.chunk_len;
+    const float dec = a.decay[h];
+    const size_t step = (size_t)a.H * per_head;
+    float* cp = a.scratch + ((size_t)b * a.n_chunks * a.H + h) * per_head + e;
+    float t = cp[0];
+    for (int c = 1; c < nc; ++c) {
+        const int len = n - c * a.chunk_len < a.chunk_len ? n - c * a.chunk_len : a.chunk_len;
+        const float own = cp[c * step];
+        cp[c * step] = t;
+        t = fmaf(powf(dec, (float)len), t, own);
+    }
+    a.state[((size_t)a.slots[b] * a.H + h) * per_head + e] = t;
 }
 
 // the shape of a request's state as [H, shape[0], Dv, shape[1]]
@@ -223,7 +274,7 @@ extern "C" int xr_recurrence_state_dims(int D, int* rows, int* lanes) {
 extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, const float* v, const float* beta,
                                     const float* gate, const float* decay, float* state, const int* cu_q,
                                     const int* slots, int B, int H, int G, int D, int Dv, int ld, int ld_g, int mode,
-                                    hipStream_t stream) {
+                                    int chunk_len, int n_chunks, float* scratch, hipStream_t stream) {
     XR_REQUIRE(B >= 0 && H > 0 && G > 0 && H % G == 0, "recurrence: %d heads over %d key heads", H, G);
     XR_REQUIRE(D > 0 && D <= 256 && Dv > 0, "recurrence: key size %d (1 to 256), value size %d", D, Dv);
     XR_REQUIRE(mode == XR_REC_RETENTION || mode == XR_REC_DELTA, "recurrence: mode %d", mode);
@@ -231,9 +282,13 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
                "recurrence: the mode's gates are missing");
     XR_REQUIRE(out && q && k && v && state && cu_q && slots, "recurrence: a pointer is missing");
     if (B == 0) return XR_OK;
-    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g};
+    const bool chunks = chunk_len > 0;
+    XR_REQUIRE(!chunks || (mode == XR_REC_RETENTION && n_chunks > 1 && scratch && chunk_len % REC_TOKENS == 0),
+               "recurrence: chunks are for retention, with room for their states");
+    XR_REQUIRE(!chunks || (long long)B * n_chunks <= 65535, "recurrence: %d requests of %d chunks", B, n_chunks);
+    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g, chunks ? 1 : 0, chunk_len, n_chunks, scratch};
     const int R = rec_lanes(D), cols = 256 / R, per = (D + R - 1) / R;
-    dim3 grid((Dv + cols - 1) / cols, H, B);
+    dim3 grid((Dv + cols - 1) / cols, H, chunks ? B * n_chunks : B);
 #define REC(M)                                                                          \
     do {                                                                                \
         if (R == 4) k_recurrence<M, 4, 8><<<grid, 256, 0, stream>>>(a);                 \
@@ -243,6 +298,12 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
     } while (0)
     if (mode == XR_REC_DELTA) REC(XR_REC_DELTA);
     else REC(XR_REC_RETENTION);
+    if (chunks) {
+        const int per_head = per * Dv * R;
+        k_retention_carry<<<dim3((per_head + 255) / 256, H, B), 256, 0, stream>>>(a, per_head);
+        a.pass = 2;
+        REC(XR_REC_RETENTION);
+    }
 #undef REC
     XR_CHECK_LAUNCH("linear_recurrence");
     return XR_OK;
