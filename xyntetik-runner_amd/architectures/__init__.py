@@ -1,2 +1,3 @@
 from . import llama    # noqa: F401  (registers LlamaForCausalLM)
 from . import suripel    # noqa: F401  (registers Suripel)
+from . import sugosun    # noqa: F401  (registers Sugosun)

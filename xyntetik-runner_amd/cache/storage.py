@@ -39,7 +39,7 @@ class CacheStorage:
     def __init__(self, kv_specs: List[Optional[KVSpec]], state_specs: List[Optional[StateSpec]],
                  cache_of: List[Optional[int]], page_size: int,
                  pages_per_group: Union[int, Callable[[KVSpec], int]], n_slots: int,
-                 dtype: torch.dtype, device: torch.device):
+                 dtype: torch.dtype, device: torch.device, model_states: Optional[Dict[str, StateSpec]] = None):
         """``kv_specs[i]``/``state_specs[i]``/``cache_of[i]`` describe entry ``i`` of the run order.
         ``pages_per_group``: one number for every group, or a function of a group's ``KVSpec``
         (a group that keeps a window of keys needs fewer pages than one that keeps them all)."""
@@ -66,6 +66,9 @@ class CacheStorage:
             named = {} if st is None else ({"mixer": st} if isinstance(st, StateSpec) else dict(st))
             return {name: torch.zeros((n_slots + 1,) + tuple(s.shape), dtype=s.dtype or dtype, device=device)
                     for name, s in named.items()}
+
+        # per-request state that belongs to no layer (an embedding's, say), by name
+        self.model_states: Dict[str, torch.Tensor] = states_of(dict(model_states) if model_states else None)
 
         for i, (kv, st) in enumerate(zip(kv_specs, state_specs)):
             owner = cache_of[i]

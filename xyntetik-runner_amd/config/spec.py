@@ -42,6 +42,7 @@ class LayerSpec:
     norms: Mapping[str, PartSpec] = field(default_factory=dict)
     block: str = "prenorm"
     filters: Mapping[str, PartSpec] = field(default_factory=dict)    # sequence filters, by the arrangement's names
+    connections: Mapping[str, PartSpec] = field(default_factory=dict)    # how sublayers meet the residual streams, likewise
 
 
 @dataclass(frozen=True)
@@ -70,8 +71,11 @@ class ModelSpec:
     head: PartSpec
     eos_token_ids: tuple = ()
     bos_token_id: Optional[int] = None
+    streams: Optional[int] = None       # copies of the residual stream the layers keep (None: the one stream)
 
     def validate(self) -> None:
+        if self.streams is not None and self.streams < 1:
+            raise ValueError(f"a model has at least one residual stream, not {self.streams}")
         for i, st in enumerate(self.order):
             if not (0 <= st.layer < len(self.layers)):
                 raise ValueError(f"run order entry {i} names layer {st.layer}, model has {len(self.layers)}")

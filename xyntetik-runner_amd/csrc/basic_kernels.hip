@@ -325,25 +325,28 @@ extern "C" int xr_rope_kv_write(const float* q_in, const float* k_in, const floa
 // h = act(g) * u; act = SiLU: g / (1 + exp(-g)) (src/model.c:4451-4452,
 // src/kernels.cu:2868-2874).  gu row = [gate(F) | up(F)].
 template <typename TI, typename TO>
-__global__ void k_gate_mul(TO* __restrict__ out, const TI* __restrict__ gu, int F, int ld_gu, size_t n, int act) {
+__global__ void k_gate_mul(TO* __restrict__ out, const TI* __restrict__ gu, int F, int ld_gu, size_t n, int act, float param) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     size_t t = i / F;
     int c = (int)(i - t * F);
     float g = ld<TI>(gu, t * ld_gu + c);
     float u = ld<TI>(gu, t * ld_gu + F + c);
-    st<TO>(out, i, gate_act<false>(act, g) * u);
+    st<TO>(out, i, gated_value(act, param, g, u));
 }
 
-extern "C" int xr_gate_mul(void* out, const void* gu, int T, int F, int ld_gu, int dtype, int act, hipStream_t stream) {
+// dtype: of gu; out_dtype: of out (32-bit branches may leave as bfloat16)
+extern "C" int xr_gate_mul(void* out, const void* gu, int T, int F, int ld_gu, int dtype, int out_dtype, int act, float param,
+                           hipStream_t stream) {
     XR_REQUIRE(T >= 0 && F > 0 && ld_gu >= 2 * F, "gate_mul: bad sizes T=%d F=%d ld=%d", T, F, ld_gu);
-    XR_REQUIRE(act >= 0 && act < XR_ACT_COUNT, "gate_mul: unknown activation code %d", act);
+    XR_REQUIRE(act >= 0 && act < XR_GATE_COUNT, "gate_mul: unknown activation code %d", act);
     size_t n = (size_t)T * F;
     if (n == 0) return XR_OK;
     unsigned blocks = (unsigned)((n + 255) / 256);
-    if (dtype == XR_F32) k_gate_mul<float, float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, F, ld_gu, n, act);
-    else if (dtype == XR_BF16) k_gate_mul<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, F, ld_gu, n, act);
-    else { xr_set_error("gate_mul: bad dtype %d", dtype); return XR_BAD_ARG; }
+    if (dtype == XR_F32 && out_dtype == XR_F32) k_gate_mul<float, float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, F, ld_gu, n, act, param);
+    else if (dtype == XR_F32 && out_dtype == XR_BF16) k_gate_mul<float, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const float*)gu, F, ld_gu, n, act, param);
+    else if (dtype == XR_BF16 && out_dtype == XR_BF16) k_gate_mul<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, F, ld_gu, n, act, param);
+    else { xr_set_error("gate_mul: bad dtypes %d -> %d", dtype, out_dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("gate_mul");
     return XR_OK;
 }

@@ -93,6 +93,26 @@ template <bool FAST> __device__ inline float gate_act(int act, float g) {
 template <bool FAST> __host__ __device__ inline float gate_act(int, float g) { return g; }   // the host pass only parses the callers
 #endif
 
+// A gated feed-forward's value from its two branches, for gates that also shape the other branch
+// and take a number of their own.  Codes below XR_ACT_COUNT are act(gate) * up as above (the
+// products' epilogues apply those themselves); the others are applied by k_gate_mul alone.
+// XR_GATE_CLAMPED_SWISH with limit L: g' = min(g, L), u' = clamp(u, -L, L),
+// value = g' sigmoid(1.702 g') (u' + 1).
+#define XR_GATE_CLAMPED_SWISH 1
+#define XR_GATE_COUNT 2
+#if defined(__HIP_DEVICE_COMPILE__)
+__device__ inline float gated_value(int act, float param, float g, float u) {
+    if (act == XR_GATE_CLAMPED_SWISH) {
+        g = fminf(g, param);
+        u = fminf(fmaxf(u, -param), param);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return gate_act<false>(act, g) * u;
+}
+#else
+__host__ __device__ inline float gated_value(int, float, float g, float u) { return g * u; }   // the host pass only parses the callers
+#endif
+
 template <typename T> __device__ inline float ld(const T* p, size_t i);
 template <> __device__ inline float ld<float>(const float* p, size_t i) { return p[i]; }
 template <> __device__ inline float ld<bf16_t>(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }

@@ -1,0 +1,142 @@
+// A feed-forward of many small experts of which every token uses a few ("mixture of experts").
+//
+// k_moe_route: per token the router's logits in 32 bits, a softmax over all experts, the `top`
+// experts with the largest score + correction (ties: the lower index), and their weights: the
+// chosen scores (without the correction) over their sum + 1e-20.
+// k_moe_up / k_moe_down: the experts' two products token by token, a wave an output column, the
+// weights of the chosen experts streamed: what a few decoded tokens need.  Expert:
+// down(act(up h)), act = relu squared.  The down product adds a token's experts up in the order
+// of its choice and writes (or adds to) 32-bit rows.
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 1024
+#define MOE_MAX_TOP 16
+
+template <typename TH>
+__global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* __restrict__ wts, const TH* __restrict__ h,
+                                                  const float* __restrict__ router, const float* __restrict__ correction,
+                                                  int E, int ld_h, int n, int top) {
+    __shared__ float z[MOE_MAX_EXPERTS];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const TH* row = h + (size_t)t * ld_h;
+    for (int e = 0; e < n; ++e) {
+        const float* w = router + (size_t)e * E;
+        float a = 0.f;
+        for (int i = lane; i < E; i += 64) a += ld<TH>(row, i) * w[i];
+        a = wave_sum(a);
+        if (lane == 0) z[e] = a;
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int e = lane; e < n; e += 64) m = fmaxf(m, z[e]);
+    m = wave_max(m);
+    float l = 0.f;
+    for (int e = lane; e < n; e += 64) l += expf(z[e] - m);
+    l = wave_sum(l);
+    __syncthreads();
+    for (int e = lane; e < n; e += 64) z[e] = expf(z[e] - m) / l;       // the scores
+    __syncthreads();
+    // `top` rounds of: the largest score + correction not yet taken, the lower index on a tie
+    float total = 0.f;
+    int mine = -1;          // lane j keeps the j-th choice
+    float mine_s = 0.f;
+    for (int j = 0; j < top; ++j) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int e = lane; e < n; e += 64) {
+            const float s = z[e];
+            if (s >= 0.f) {                 // a taken score is stored as -(s) - 1, which is negative
+                const float c = s + correction[e];
+                if (c > best || (c == best && e < at)) { best = c; at = e; }
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, 64);
+            const int oa = __shfl_xor(at, o, 64);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+        const float s = z[at];
+        total += s;
+        if (lane == j) { mine = at; mine_s = s; }
+        __syncthreads();
+        if (lane == 0) z[at] = -s - 1.0f;
+        __syncthreads();
+    }
+    if (lane < top) {
+        idx[(size_t)t * top + lane] = mine;
+        wts[(size_t)t * top + lane] = mine_s / (total + 1e-20f);
+    }
+}
+
+extern "C" int xr_moe_route(int* idx, float* wts, const void* h, const float* router, const float* correction, int T, int E,
+                            int ld_h, int n, int top, int h_dtype, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && E > 0 && ld_h >= E, "moe_route: bad sizes T=%d E=%d ld=%d", T, E, ld_h);
+    XR_REQUIRE(n >= 1 && n <= MOE_MAX_EXPERTS && top >= 1 && top <= n && top <= MOE_MAX_TOP,
+               "moe_route: %d experts (at most %d), %d chosen (at most %d)", n, MOE_MAX_EXPERTS, top, MOE_MAX_TOP);
+    if (T == 0) return XR_OK;
+    if (h_dtype == XR_F32) k_moe_route<float><<<T, 64, 0, stream>>>(idx, wts, (const float*)h, router, correction, E, ld_h, n, top);
+    else if (h_dtype == XR_BF16) k_moe_route<bf16_t><<<T, 64, 0, stream>>>(idx, wts, (const bf16_t*)h, router, correction, E, ld_h, n, top);
+    else { xr_set_error("moe_route: bad dtype %d", h_dtype); return XR_BAD_ARG; }
+    XR_CHECK_LAUNCH("moe_route");
+    return XR_OK;
+}
+
+// z[t * top + j][f] = relu(W_up[e][f] . h[t])^2 for e = idx[t][j].  Grid (T * top, ceil(F / 4)); a wave a column.
+template <typename TW>
+__global__ __launch_bounds__(256) void k_moe_up(TW* __restrict__ z, const TW* __restrict__ h, const TW* __restrict__ w_up,
+                                                const int* __restrict__ idx, int E, int F, int ld_h, int top) {
+    const int a = blockIdx.x, f = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (f >= F) return;
+    const int t = a / top, e = idx[a];
+    const TW* row = h + (size_t)t * ld_h;
+    const TW* w = w_up + ((size_t)e * F + f) * E;
+    float acc = 0.f;
+    for (int i = lane; i < E; i += 64) acc += ld<TW>(w, i) * ld<TW>(row, i);
+    acc = wave_sum(acc);
+    if (lane == 0) {
+        const float r = fmaxf(acc, 0.f);
+        st<TW>(z, (size_t)a * F + f, r * r);
+    }
+}
+
+// y[t][c] (+)= sum_j wts[t][j] * (W_down[e_j][c] . z[t * top + j]).  Grid (T, ceil(E / 4)); a wave a column.
+template <typename TW>
+__global__ __launch_bounds__(256) void k_moe_down(float* __restrict__ y, const TW* __restrict__ z, const TW* __restrict__ w_down,
+                                                  const int* __restrict__ idx, const float* __restrict__ wts, int E, int F,
+                                                  int ld_y, int top, int accumulate) {
+    const int t = blockIdx.x, c = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (c >= E) return;
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) {
+        const int e = idx[(size_t)t * top + j];
+        const TW* w = w_down + ((size_t)e * E + c) * F;
+        const TW* zr = z + ((size_t)t * top + j) * F;
+        float acc = 0.f;
+        for (int i = lane; i < F; i += 64) acc += ld<TW>(w, i) * ld<TW>(zr, i);
+        sum += wts[(size_t)t * top + j] * wave_sum(acc);
+    }
+    if (lane == 0) {
+        float* o = y + (size_t)t * ld_y + c;
+        *o = accumulate ? *o + sum : sum;
+    }
+}
+
+extern "C" int xr_moe_experts(float* y, void* z, const void* h, const void* w_up, const void* w_down, const int* idx,
+                              const float* wts, int T, int E, int F, int ld_h, int ld_y, int n, int top, int accumulate,
+                              int dtype, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && E > 0 && F > 0 && ld_h >= E && ld_y >= E, "moe_experts: bad sizes T=%d E=%d F=%d", T, E, F);
+    XR_REQUIRE(n >= 1 && top >= 1 && top <= n && top <= MOE_MAX_TOP, "moe_experts: %d experts, %d chosen", n, top);
+    XR_REQUIRE((long long)T * top <= 0x7fffffffLL, "moe_experts: too many rows");
+    if (T == 0) return XR_OK;
+    const dim3 gu(T * top, (F + 3) / 4), gd(T, (E + 3) / 4);
+    if (dtype == XR_F32) {
+        k_moe_up<float><<<gu, 256, 0, stream>>>((float*)z, (const float*)h, (const float*)w_up, idx, E, F, ld_h, top);
+        k_moe_down<float><<<gd, 256, 0, stream>>>(y, (const float*)z, (const float*)w_down, idx, wts, E, F, ld_y, top, accumulate);
+    } else if (dtype == XR_BF16) {
+        k_moe_up<bf16_t><<<gu, 256, 0, stream>>>((bf16_t*)z, (const bf16_t*)h, (const bf16_t*)w_up, idx, E, F, ld_h, top);
+        k_moe_down<bf16_t><<<gd, 256, 0, stream>>>(y, (const bf16_t*)z, (const bf16_t*)w_down, idx, wts, E, F, ld_y, top, accumulate);
+    } else { xr_set_error("moe_experts: bad dtype %d", dtype); return XR_BAD_ARG; }
+    XR_CHECK_LAUNCH("moe_experts");
+    return XR_OK;
+}

@@ -20,6 +20,10 @@ XR_F32, XR_BF16 = 0, 1
 _CODE = {torch.float32: XR_F32, torch.bfloat16: XR_BF16}
 # activations of a gated feed-forward, by the code the kernels know them under (XR_ACT_* of common.h)
 GATE_ACTIVATIONS = {"silu": 0}
+# gates that also shape the other branch and take a number of their own (XR_GATE_* of common.h): applied by
+# ``gate_mul`` to the 32-bit result of the gate-and-up product, not by the product's epilogue
+SHAPED_GATES = {"clamped_swish": 1}
+NORM_GATES = {"silu": 0, "sigmoid": 1}                  # XR_GATE_SILU / XR_GATE_SIGMOID of sequence_kernels.hip
 
 
 class KernelError(RuntimeError):
@@ -46,7 +50,7 @@ _PROTOS = {
     "xr_embedding": [_p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rope_kv_write": [_p, _p, _p, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
-    "xr_gate_mul": [_p, _p, _i, _i, _i, _i, _i, _p],
+    "xr_gate_mul": [_p, _p, _i, _i, _i, _i, _i, _i, _f, _p],
     "xr_add": [_p, _p, _sz, _i, _p],
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_fill_rows_many": [_p, _p, _i, _sz, _p, _i, _u32, _p],
@@ -63,7 +67,15 @@ _PROTOS = {
     "xr_causal_conv": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_polynorm": [_p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rotate_rows": [_p, _p, _p, _i, _i, _i, _i, _i, _f, _p],
-    "xr_gated_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _p],
+    "xr_gated_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _i, _p],
+    "xr_act_rows": [_p, _i, _i, _i, _i, _p],
+    "xr_embedding_pairs": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p],
+    "xr_streams_expand": [_p, _p, _i, _i, _i, _p],
+    "xr_streams_sum": [_p, _p, _i, _i, _i, _p],
+    "xr_streams_step": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
+    "xr_latent_prepare": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p],
+    "xr_moe_route": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p],
+    "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
     "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p],
     "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
@@ -229,16 +241,21 @@ class Ops:
                                            dtype_code(w.dtype) if w is not None else XR_F32, _stream()))
         return out
 
-    def gate_mul(self, gu: torch.Tensor, activation: str = "silu") -> torch.Tensor:
-        """``act(gu[:, :F]) * gu[:, F:]``."""
+    def gate_mul(self, gu: torch.Tensor, activation: str = "silu", param: float = 0.0,
+                 out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """``act(gu[:, :F]) * gu[:, F:]`` for a gate of ``GATE_ACTIVATIONS``; for one of ``SHAPED_GATES`` the
+        value the gate makes of both branches with its number ``param`` ("clamped_swish" with limit L:
+        ``g' = min(g, L)``, ``u' = clamp(u, -L, L)``, ``g' sigmoid(1.702 g') (u' + 1)``).  32-bit branches may
+        leave in ``out_dtype``."""
         self._dev(gu)
         T, F2 = gu.shape
         F = F2 // 2
         if gu.stride(1) != 1 or F2 % 2:
             raise KernelError("gate_mul input must be [rows, 2F] with unit column stride")
-        out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
-        self.lib.check(self.lib.xr_gate_mul(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0),
-                                            dtype_code(gu.dtype), activation_code(activation), _stream()))
+        code = SHAPED_GATES[activation] if activation in SHAPED_GATES else activation_code(activation)
+        out = torch.empty((T, F), dtype=out_dtype or gu.dtype, device=gu.device)
+        self.lib.check(self.lib.xr_gate_mul(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0), dtype_code(gu.dtype),
+                                            dtype_code(out.dtype), code, float(param), _stream()))
         return out
 
     def silu_mul(self, gu: torch.Tensor) -> torch.Tensor:
@@ -438,10 +455,14 @@ class Ops:
         return self.rmsnorm(residual, norm_weight, eps, out_dtype)
 
     def linear_gated(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None, activation: str = "silu",
-                     variant: int = 0) -> torch.Tensor:
+                     variant: int = 0, param: float = 0.0) -> torch.Tensor:
         """``act(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows
         (a matrix, or a ``PackedWeight`` made with ``gated=True``); ``activation`` is one of
-        ``GATE_ACTIVATIONS``."""
+        ``GATE_ACTIVATIONS``, or one of ``SHAPED_GATES`` with its number ``param`` (the product then leaves
+        both branches in 32 bits and ``gate_mul`` makes the value of them)."""
+        if activation in SHAPED_GATES:
+            rows = a.data if isinstance(a, UnscaledRows) else a
+            return self.gate_mul(self.linear(a, w, bias=bias, out_dtype=torch.float32), activation, param, out_dtype=rows.dtype)
         act = activation_code(activation)
         packed = isinstance(w, PackedWeight)
         wt = w.data if packed else w
@@ -708,20 +729,196 @@ class Ops:
                                                rot, x.stride(0), float(scale), _stream()))
 
     def gated_rmsnorm(self, o: torch.Tensor, gate: torch.Tensor, w: Optional[torch.Tensor], H: int, Dv: int, eps: float,
-                      out_dtype: torch.dtype) -> torch.Tensor:
-        """``o / rms(o) * w * silu(gate)`` per head: ``o [T, H * Dv]`` 32-bit and contiguous, ``gate`` a
-        32-bit view of the same shape, ``w [Dv]`` 32-bit or absent."""
+                      out_dtype: torch.dtype, gate_activation: str = "silu") -> torch.Tensor:
+        """``o / rms(o) * w * act(gate)`` per head: ``o [T, H * Dv]`` 32-bit and contiguous, ``gate`` a
+        32-bit view of the same shape; ``w`` 32-bit: ``[Dv]`` (the heads share it), ``[H * Dv]`` (one a
+        channel of the row) or absent; ``act`` "silu" or "sigmoid".  A norm over all heads together is
+        ``H = 1`` with ``Dv`` the whole row."""
         self._dev(o, gate, w)
         T = o.shape[0]
         if o.dtype != torch.float32 or not o.is_contiguous() or o.shape[1] != H * Dv:
             raise KernelError(f"gated_rmsnorm: o must be contiguous float32 [rows, {H * Dv}]")
         if gate.dtype != torch.float32 or gate.stride(1) != 1 or tuple(gate.shape) != (T, H * Dv):
             raise KernelError("gated_rmsnorm: the gate must be a float32 view of o's shape")
-        if w is not None and (w.dtype != torch.float32 or w.numel() != Dv):
-            raise KernelError(f"gated_rmsnorm: the weight must be float32 [{Dv}]")
+        if w is not None and (w.dtype != torch.float32 or w.numel() not in (Dv, H * Dv) or not w.is_contiguous()):
+            raise KernelError(f"gated_rmsnorm: the weight must be float32 [{Dv}] or [{H * Dv}]")
+        if gate_activation not in NORM_GATES:
+            raise KernelError(f"gated_rmsnorm: gate activation {gate_activation!r} (known: {sorted(NORM_GATES)})")
         out = torch.empty((T, H * Dv), dtype=out_dtype, device=o.device)
         self.lib.check(self.lib.xr_gated_rmsnorm(out.data_ptr(), o.data_ptr(), gate.data_ptr(), _ptr(w), T, H, Dv,
-                                                 gate.stride(0), float(eps), dtype_code(out_dtype), _stream()))
+                                                 gate.stride(0), float(eps), dtype_code(out_dtype),
+                                                 1 if (w is not None and H > 1 and w.numel() == H * Dv) else 0,
+                                                 NORM_GATES[gate_activation], _stream()))
+        return out
+
+    def act_rows_(self, x: torch.Tensor, activation: str = "silu") -> None:
+        """``x <- act(x)`` in place on a 32-bit view ``[rows, width]`` with unit column stride."""
+        self._dev(x)
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+            raise KernelError("act_rows_: x must be a float32 view [rows, width] with unit column stride")
+        if activation != "silu":
+            raise KernelError(f"act_rows_: activation {activation!r} is not built (silu)")
+        self.lib.check(self.lib.xr_act_rows(x.data_ptr(), x.shape[0], x.shape[1], x.stride(0), CONV_ACTIVATIONS[activation], _stream()))
+
+    # -- an embedding with a hashed table of token pairs --------------------------
+    def embedding_pairs(self, table: torch.Tensor, pairs: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], ids, ctx,
+                        last_token: Optional[torch.Tensor], buckets: int, mul_prev: int, mul_cur: int, eps: float) -> torch.Tensor:
+        """``rmsnorm(table[id] + pairs[(prev * mul_prev + id * mul_cur) % buckets]) * norm_w`` as 32-bit rows
+        (``pairs`` absent: the token's row alone; ``norm_w`` absent: no norm).  The token at position 0 reads
+        row ``buckets`` of ``pairs [buckets + 1, E]``.  ``last_token [slots + 1]`` (int32) holds every request's
+        last token of the step before and is brought up to date; ``ctx`` gives the step's rows."""
+        self._dev(table, pairs, norm_w, ids, last_token)
+        self._contig(table, "embedding table")
+        V, E = table.shape
+        if pairs is not None:
+            self._contig(pairs, "pair table")
+            if pairs.dtype != table.dtype or tuple(pairs.shape) != (buckets + 1, E):
+                raise KernelError(f"embedding_pairs: the pair table must be {table.dtype} [{buckets + 1}, {E}]")
+            if last_token is None or last_token.dtype != torch.int32 or not last_token.is_contiguous():
+                raise KernelError("embedding_pairs: the requests' last tokens must be int32 [slots]")
+        if norm_w is not None and (norm_w.dtype != torch.float32 or norm_w.numel() != E or not norm_w.is_contiguous()):
+            raise KernelError(f"embedding_pairs: the norm's weight must be float32 [{E}]")
+        T = ids.numel()
+        out = torch.empty((T, E), dtype=torch.float32, device=table.device)
+        self.lib.check(self.lib.xr_embedding_pairs(out.data_ptr(), table.data_ptr(), _ptr(pairs), _ptr(norm_w), ids.data_ptr(),
+                                                   ctx.positions.data_ptr(), ctx.req_of_token.data_ptr(), ctx.cu_q.data_ptr(),
+                                                   ctx.slots.data_ptr(), _ptr(last_token), T, E, V, int(buckets), int(mul_prev),
+                                                   int(mul_cur), float(eps), dtype_code(table.dtype), _stream()))
+        return out
+
+    # -- several copies of the residual stream -------------------------------------
+    MAX_STREAMS = 8
+
+    def streams_expand(self, x: torch.Tensor, S: int) -> torch.Tensor:
+        """``[S, T, E]``: ``S`` copies of the 32-bit rows ``x [T, E]``."""
+        self._dev(x)
+        if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
+            raise KernelError("streams_expand: x must be contiguous float32 [rows, width]")
+        xs = torch.empty((S,) + tuple(x.shape), dtype=torch.float32, device=x.device)
+        self.lib.check(self.lib.xr_streams_expand(xs.data_ptr(), x.data_ptr(), x.shape[0], x.shape[1], int(S), _stream()))
+        return xs
+
+    def streams_sum(self, xs: torch.Tensor) -> torch.Tensor:
+        """The sum ``[T, E]`` of the copies ``xs [S, T, E]``."""
+        self._dev(xs)
+        if xs.dtype != torch.float32 or xs.dim() != 3 or not xs.is_contiguous():
+            raise KernelError("streams_sum: xs must be contiguous float32 [streams, rows, width]")
+        x = torch.empty(tuple(xs.shape[1:]), dtype=torch.float32, device=xs.device)
+        self.lib.check(self.lib.xr_streams_sum(x.data_ptr(), xs.data_ptr(), xs.shape[1], xs.shape[2], xs.shape[0], _stream()))
+        return x
+
+    def streams_step(self, xs: torch.Tensor, y: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                     out_w: Optional[torch.Tensor] = None, in_w: Optional[torch.Tensor] = None,
+                     norm_w: Optional[torch.Tensor] = None, eps: float = 0.0,
+                     h_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+        """One pass over the copies ``xs [S, T, E]`` around a sublayer.  With ``y [T, E]`` (32-bit), all
+        copies at once from the old ones: ``xs_t <- sum_s mix[s, t] xs_s + out_w[t] y``.  With ``in_w``, then:
+        ``u = sum_s in_w[s] xs_s`` and its RMSNorm times ``norm_w`` comes back in ``h_dtype`` (``norm_w``
+        absent: ``u`` itself).  Weights are 32-bit."""
+        self._dev(xs, y, mix, out_w, in_w, norm_w)
+        if xs.dtype != torch.float32 or xs.dim() != 3 or not xs.is_contiguous():
+            raise KernelError("streams_step: xs must be contiguous float32 [streams, rows, width]")
+        S, T, E = xs.shape
+        if S > self.MAX_STREAMS:
+            raise KernelError(f"streams_step: {S} streams (the kernel takes up to {self.MAX_STREAMS})")
+        if y is not None:
+            if y.dtype != torch.float32 or tuple(y.shape) != (T, E) or not y.is_contiguous():
+                raise KernelError(f"streams_step: y must be contiguous float32 [{T}, {E}]")
+            if (mix is None or out_w is None or mix.dtype != torch.float32 or out_w.dtype != torch.float32
+                    or tuple(mix.shape) != (S, S) or out_w.numel() != S or not mix.is_contiguous()):
+                raise KernelError(f"streams_step: the write needs float32 mix [{S}, {S}] and out [{S}]")
+        h = None
+        if in_w is not None:
+            if in_w.dtype != torch.float32 or in_w.numel() != S:
+                raise KernelError(f"streams_step: the read needs float32 in [{S}]")
+            if norm_w is not None and (norm_w.dtype != torch.float32 or norm_w.numel() != E or not norm_w.is_contiguous()):
+                raise KernelError(f"streams_step: the norm's weight must be float32 [{E}]")
+            h = torch.empty((T, E), dtype=h_dtype or torch.float32, device=xs.device)
+        self.lib.check(self.lib.xr_streams_step(xs.data_ptr(), _ptr(y), _ptr(mix), _ptr(out_w), _ptr(in_w), _ptr(norm_w), _ptr(h),
+                                                T, E, S, float(eps), dtype_code(h.dtype) if h is not None else XR_F32, _stream()))
+        return h
+
+    # -- latent attention ------------------------------------------------------------
+    def latent_prepare(self, q_in: torch.Tensor, kv_in: torch.Tensor, c_w: torch.Tensor, eps: float, q_out: torch.Tensor,
+                       k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, group: int, inv_freq: Optional[torch.Tensor],
+                       H: int, D: int, R: int, C: int, dims: int, page_size: int) -> torch.Tensor:
+        """Between a latent attention's down projections and its attention.  ``q_in [T, H * (D + R)]`` and
+        ``kv_in [T, C + R]`` are 32-bit views.  The first ``C`` channels of ``kv_in`` are normed (RMS, weight
+        ``c_w``) into the latent; the last ``R`` are the shared key part, whose first ``dims`` channels are
+        rotated in pairs ``(2i, 2i + 1)`` by position x ``inv_freq[i]``, as are the last ``R`` channels of every
+        query head.  The row ``[latent | key part]`` goes to the key pages ``[pages, 1, page, C + R]`` and,
+        transposed, to the value pages ``[pages, 1, C or C + R, page]``; the rotated query channels go to
+        ``q_out[:, h, C:]`` (``q_out [T, H * (C + R)]``); the unrotated ones come back ``[T, H * D]`` in
+        ``q_out``'s dtype."""
+        self._dev(q_in, kv_in, c_w, q_out, k_cache, v_cache, inv_freq)
+        T = q_in.shape[0]
+        if any(t.dtype != torch.float32 or t.stride(1) != 1 for t in (q_in, kv_in)):
+            raise KernelError("latent_prepare: q and kv inputs must be float32 views with unit column stride")
+        if tuple(q_in.shape) != (T, H * (D + R)) or tuple(kv_in.shape) != (T, C + R):
+            raise KernelError("latent_prepare: input widths do not fit the heads")
+        if c_w.dtype != torch.float32 or c_w.numel() != C or not c_w.is_contiguous():
+            raise KernelError(f"latent_prepare: the latent norm's weight must be float32 [{C}]")
+        dt = q_out.dtype
+        if tuple(q_out.shape) != (T, H * (C + R)) or not q_out.is_contiguous():
+            raise KernelError(f"latent_prepare: the query output must be contiguous [{T}, {H * (C + R)}]")
+        Dvc = v_cache.shape[2]
+        if (k_cache.dtype != dt or v_cache.dtype != dt or tuple(k_cache.shape[1:]) != (1, page_size, C + R)
+                or tuple(v_cache.shape[1:]) != (1, Dvc, page_size) or Dvc not in (C, C + R)):
+            raise KernelError("latent_prepare: the cache does not fit one key/value head of the latent's row")
+        if dims and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != dims // 2):
+            raise KernelError(f"latent_prepare: {dims // 2} 32-bit frequencies are needed")
+        table = ctx.block_table(group)
+        qn = torch.empty((T, H * D), dtype=dt, device=q_in.device)
+        self.lib.check(self.lib.xr_latent_prepare(qn.data_ptr(), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                  q_in.data_ptr(), kv_in.data_ptr(), c_w.data_ptr(), ctx.positions.data_ptr(),
+                                                  ctx.req_of_token.data_ptr(), table.data_ptr(), table.stride(0), _ptr(inv_freq),
+                                                  T, H, D, R, C, Dvc, int(dims), q_in.stride(0), kv_in.stride(0), page_size,
+                                                  float(eps), dtype_code(dt), _stream()))
+        return qn
+
+    # -- mixture of experts ------------------------------------------------------------
+    def moe_route(self, h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int):
+        """``(experts [T, top] int32, weights [T, top] float32)``: 32-bit logits ``router [n, E] @ h``, a softmax
+        over all experts, the ``top`` largest of score + ``correction`` (the lower index on a tie), weights =
+        the chosen scores over their sum + 1e-20."""
+        self._dev(h, router, correction)
+        if h.dim() != 2 or h.stride(1) != 1:
+            raise KernelError("moe_route: h must be [rows, width] with unit column stride")
+        T, E = h.shape
+        n = router.shape[0]
+        if (router.dtype != torch.float32 or tuple(router.shape) != (n, E) or not router.is_contiguous()
+                or correction.dtype != torch.float32 or correction.numel() != n):
+            raise KernelError(f"moe_route: router must be float32 [{n}, {E}] and the correction float32 [{n}]")
+        idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
+        wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
+        self.lib.check(self.lib.xr_moe_route(idx.data_ptr(), wts.data_ptr(), h.data_ptr(), router.data_ptr(), correction.data_ptr(),
+                                             T, E, h.stride(0), n, int(top), dtype_code(h.dtype), _stream()))
+        return idx, wts
+
+    def moe_experts(self, h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor,
+                    out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+        """``out[t] (+)= sum_j wts[t, j] * w_down[e] @ relu(w_up[e] @ h[t])^2`` with ``e = idx[t, j]``, as 32-bit
+        rows; ``w_up [n, F, E]`` and ``w_down [n, E, F]`` in ``h``'s dtype."""
+        self._dev(h, w_up, w_down, idx, wts, out)
+        T, E = h.shape
+        n, F, _ = w_up.shape
+        top = idx.shape[1]
+        if h.stride(1) != 1 or w_up.dtype != h.dtype or w_down.dtype != h.dtype:
+            raise KernelError("moe_experts: h must have unit column stride and the experts its dtype")
+        if tuple(w_up.shape) != (n, F, E) or tuple(w_down.shape) != (n, E, F) or not w_up.is_contiguous() or not w_down.is_contiguous():
+            raise KernelError("moe_experts: the experts' weights must be contiguous [n, F, E] and [n, E, F]")
+        if idx.dtype != torch.int32 or wts.dtype != torch.float32 or tuple(idx.shape) != (T, top) or tuple(wts.shape) != (T, top):
+            raise KernelError("moe_experts: the choice must be int32 [T, top] with float32 weights")
+        if out is None:
+            if accumulate:
+                raise KernelError("moe_experts: accumulate needs an output")
+            out = torch.empty((T, E), dtype=torch.float32, device=h.device)
+        elif out.dtype != torch.float32 or tuple(out.shape) != (T, E) or out.stride(1) != 1:
+            raise KernelError(f"moe_experts: the output must be float32 [{T}, {E}]")
+        z = torch.empty((T * top, F), dtype=h.dtype, device=h.device)
+        self.lib.check(self.lib.xr_moe_experts(out.data_ptr(), z.data_ptr(), h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(),
+                                               idx.data_ptr(), wts.data_ptr(), T, E, F, h.stride(0), out.stride(0), n, top,
+                                               1 if accumulate else 0, dtype_code(h.dtype), _stream()))
         return out
 
     def delta_prepare_(self, q, k, b, a, a_log, dt_bias, G: int, H: int, D: int, q_scale: float, unit_eps: float) -> None:

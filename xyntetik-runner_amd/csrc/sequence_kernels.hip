@@ -337,33 +337,61 @@ extern "C" int xr_rotate_rows(float* x, const int* positions, const float* inv_f
 }
 
 // ---------------------------------------------------------------- gated norm of a read-out
-// out[t][h][d] = o[t][h][d] / sqrt(mean_d(o^2) + eps) * w[d] * silu(gate[t][h][d]); w may be absent.
-// One wave per (token, head).
+// out[t][h][d] = o[t][h][d] / sqrt(mean_d(o^2) + eps) * w * act(gate[t][h][d]); w may be absent, is one
+// weight a channel of a head that the heads share (w [Dv]) or, with w_full, one a channel of the row
+// (w [H * Dv]); act is SiLU (gate_act 0) or the sigmoid (1).  A norm over all heads together is
+// H = 1 with Dv the whole row.  One wave per (token, head).
+#define XR_GATE_SILU 0
+#define XR_GATE_SIGMOID 1
 template <typename TO>
 __global__ __launch_bounds__(64) void k_gated_rmsnorm(TO* __restrict__ out, const float* __restrict__ o,
                                                       const float* __restrict__ gate, const float* __restrict__ w,
-                                                      int H, int Dv, int ld_g, float eps) {
+                                                      int H, int Dv, int ld_g, float eps, int w_full, int gate_act) {
     const int t = blockIdx.x, h = blockIdx.y;
     const float* orow = o + ((size_t)t * H + h) * Dv;
     const float* grow = gate + (size_t)t * ld_g + (size_t)h * Dv;
+    const float* wrow = w ? (w_full ? w + (size_t)h * Dv : w) : nullptr;
     float ss = 0.f;
     for (int d = threadIdx.x; d < Dv; d += 64) ss += orow[d] * orow[d];
     const float rinv = 1.0f / sqrtf(wave_sum(ss) / (float)Dv + eps);
     TO* dst = out + ((size_t)t * H + h) * Dv;
     for (int d = threadIdx.x; d < Dv; d += 64) {
         const float g = grow[d];
-        st<TO>(dst, d, orow[d] * rinv * (w ? w[d] : 1.f) * (g / (1.0f + expf(-g))));
+        const float sg = 1.0f / (1.0f + expf(-g));
+        st<TO>(dst, d, orow[d] * rinv * (wrow ? wrow[d] : 1.f) * (gate_act == XR_GATE_SIGMOID ? sg : g * sg));
     }
 }
 
 extern "C" int xr_gated_rmsnorm(void* out, const float* o, const float* gate, const float* w, int T, int H, int Dv,
-                                int ld_g, float eps, int out_dtype, hipStream_t stream) {
+                                int ld_g, float eps, int out_dtype, int w_full, int gate_act, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && H > 0 && Dv > 0 && ld_g >= H * Dv, "gated_rmsnorm: bad sizes T=%d H=%d Dv=%d ld=%d", T, H, Dv, ld_g);
+    XR_REQUIRE(gate_act == XR_GATE_SILU || gate_act == XR_GATE_SIGMOID, "gated_rmsnorm: unknown gate activation %d", gate_act);
     if (T == 0) return XR_OK;
-    if (out_dtype == XR_F32) k_gated_rmsnorm<float><<<dim3(T, H), 64, 0, stream>>>((float*)out, o, gate, w, H, Dv, ld_g, eps);
-    else if (out_dtype == XR_BF16) k_gated_rmsnorm<bf16_t><<<dim3(T, H), 64, 0, stream>>>((bf16_t*)out, o, gate, w, H, Dv, ld_g, eps);
+    if (out_dtype == XR_F32) k_gated_rmsnorm<float><<<dim3(T, H), 64, 0, stream>>>((float*)out, o, gate, w, H, Dv, ld_g, eps, w_full, gate_act);
+    else if (out_dtype == XR_BF16) k_gated_rmsnorm<bf16_t><<<dim3(T, H), 64, 0, stream>>>((bf16_t*)out, o, gate, w, H, Dv, ld_g, eps, w_full, gate_act);
     else { xr_set_error("gated_rmsnorm: bad dtype %d", out_dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("gated_rmsnorm");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- an activation on 32-bit rows, in place
+// x[t][c] <- act(x[t][c]) for the first W columns of rows of stride ld; act 1 = SiLU.
+__global__ void k_act_rows(float* __restrict__ x, int W, int ld, size_t n, int act) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / W;
+    float* p = x + t * ld + (i - t * W);
+    const float v = *p;
+    *p = v / (1.0f + expf(-v));
+}
+
+extern "C" int xr_act_rows(float* x, int T, int W, int ld, int act, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && W > 0 && ld >= W, "act_rows: bad sizes T=%d W=%d ld=%d", T, W, ld);
+    XR_REQUIRE(act == XR_CONV_SILU, "act_rows: activation %d is not built (1 = SiLU)", act);
+    const size_t n = (size_t)T * W;
+    if (n == 0) return XR_OK;
+    k_act_rows<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, W, ld, n, act);
+    XR_CHECK_LAUNCH("act_rows");
     return XR_OK;
 }
 

@@ -27,10 +27,13 @@ class Model:
                 make_part("mixer", ls.mixer) if ls.mixer is not None else None,
                 make_part("feed_forward", ls.feed_forward) if ls.feed_forward is not None else None,
                 {name: make_part("norm", ps) for name, ps in ls.norms.items()},
-                {name: make_part("filter", ps) for name, ps in ls.filters.items()}))
+                {name: make_part("filter", ps) for name, ps in ls.filters.items()},
+                {name: make_part("connection", ps) for name, ps in ls.connections.items()}))
         self.final_norm = make_part("norm", spec.final_norm)
         self.head = make_part("head", spec.head)
         self.rt: Optional[Runtime] = None
+        self.embedding_state: Optional[torch.Tensor] = None
+        self.tap = None      # a callable (run-order entry, residual stream after it), for looking inside a step
 
     # ------------------------------------------------------------------ tensors
     def _named_parts(self):
@@ -40,6 +43,8 @@ class Model:
                 yield ps.prefix, blk.norms[name]
             for name, ps in ls.filters.items():
                 yield ps.prefix, blk.filters[name]
+            for name, ps in ls.connections.items():
+                yield ps.prefix, blk.connections[name]
             if ls.mixer is not None:
                 yield ls.mixer.prefix, blk.mixer
             if ls.feed_forward is not None:
@@ -96,10 +101,24 @@ class Model:
             of.append(step.cache_of)
         return kv, st, of
 
+    def model_states(self):
+        """Per-request state that belongs to no layer, by name: the embedding's, if it keeps any."""
+        spec = getattr(self.embedding, "state_spec", lambda: None)()
+        return {"embedding": spec} if spec is not None else {}
+
+    def attach_states(self, states) -> None:
+        """The tensors ``[slots + 1, *shape]`` the cache storage made for ``model_states()``."""
+        self.embedding_state = states.get("embedding")
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, caches) -> torch.Tensor:
         """Run the step's tokens through every layer; returns the residual stream ``[T, E]`` (32-bit)."""
-        x = self.embedding.forward(ctx, ctx.token_ids)
+        if self.embedding_state is not None:
+            x = self.embedding.forward(ctx, ctx.token_ids, state=self.embedding_state)
+        else:
+            x = self.embedding.forward(ctx, ctx.token_ids)
+        if self.spec.streams is not None:       # the layers keep several copies of the residual stream
+            x = ctx.ops.streams_expand(x, self.spec.streams)
         order = self.spec.order
         h = None            # the result of the next block's first norm, if the block before made it
         for i, step in enumerate(order):
@@ -110,6 +129,10 @@ class Model:
             else:
                 block.forward(ctx, caches[i], x)
                 h = None
+            if self.tap is not None:
+                self.tap(i, x)
+        if self.spec.streams is not None:
+            x = ctx.ops.streams_sum(x)
         return x
 
     def logits(self, ctx, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:

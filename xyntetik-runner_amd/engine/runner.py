@@ -77,7 +77,8 @@ class ModelRunner:
                                budget_bytes=memory_budget(total, free, gpu_memory_fraction, working),
                                max_model_len=max_model_len or spec.max_position)
         self.storage = CacheStorage(kv, st, of, page_size, lambda s: sizes[specs.index(s)], max_requests,
-                                    self.dtype, self.device)
+                                    self.dtype, self.device, model_states=self.model.model_states())
+        self.model.attach_states(self.storage.model_states)
         assert self.storage.group_specs == specs
         self.manager = CacheManager(specs, page_size, self.storage.group_pages, max_requests)
         self.vocab_size = spec.vocab_size
@@ -201,6 +202,7 @@ class ModelRunner:
         if not slots:
             return
         if not hasattr(self, "_fill_states"):       # every state tensor of every layer, in one launch
-            self._fill_states = self.ops.row_filler(st for lc in self.storage.layers for st in lc.states.values())
+            self._fill_states = self.ops.row_filler([st for lc in self.storage.layers for st in lc.states.values()]
+                                                    + list(self.storage.model_states.values()))
         if self._fill_states is not None:
             self._fill_states(torch.tensor(slots, dtype=torch.int32, device=self.device), len(slots), 0)

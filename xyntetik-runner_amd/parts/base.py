@@ -24,6 +24,8 @@ Families and what each must offer:
 * ``FeedForward``: ``forward(ctx, h) -> y`` and ``forward_add(ctx, h, residual)``.
 * ``SequenceFilter``: ``forward(ctx, state, h) -> h'``: what a sublayer reads passes through it on
   its way from the norm; ``state_spec()`` says what it carries from token to token.
+* ``Connection``: how a sublayer meets several copies of the residual stream: the weights that make its
+  input of them and spread its result over them.
 * ``Block``: the arrangement; it names its norms (``norm_names``), may do without a mixer or a
   feed-forward, and ``forward(ctx, cache, x)`` updates ``x`` in place.
 
@@ -182,6 +184,12 @@ class Mixer(Part):
     def forward_add(self, ctx, cache, h: torch.Tensor, residual: torch.Tensor) -> None:
         ctx.ops.add_(residual, self.forward(ctx, cache, h))
 
+    def forward_f32(self, ctx, cache, h: torch.Tensor) -> torch.Tensor:
+        """``forward`` as 32-bit rows, for an arrangement that does more with a sublayer's result than add
+        it to one residual stream.  A part whose last product can leave 32 bits overrides this; the
+        default widens what ``forward`` rounded."""
+        return ctx.ops.convert(self.forward(ctx, cache, h).contiguous(), torch.float32)
+
     def forward_add_norm(self, ctx, cache, h, residual: torch.Tensor, norm: Norm, defer: bool = False):
         """``forward_add``, then ``norm`` of the updated residual stream."""
         self.forward_add(ctx, cache, h, residual)
@@ -200,6 +208,12 @@ class SequenceFilter(Part):
         raise NotImplementedError
 
 
+class Connection(Part):
+    """How one sublayer meets ``streams`` copies of the residual stream.  A block arrangement names its
+    connections as it names its norms."""
+    streams = 1
+
+
 class FeedForward(Part):
     def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
@@ -209,6 +223,10 @@ class FeedForward(Part):
 
     def forward_add(self, ctx, h: torch.Tensor, residual: torch.Tensor) -> None:
         ctx.ops.add_(residual, self.forward(ctx, h))
+
+    def forward_f32(self, ctx, h: torch.Tensor) -> torch.Tensor:
+        """``forward`` as 32-bit rows (see ``Mixer.forward_f32``)."""
+        return ctx.ops.convert(self.forward(ctx, h).contiguous(), torch.float32)
 
     def forward_add_norm(self, ctx, h, residual: torch.Tensor, norm: Norm, defer: bool = False):
         """``forward_add``, then ``norm`` of the updated residual stream."""
@@ -224,12 +242,15 @@ class Block:
     norm_names: Tuple[str, ...] = ()
     #: the sequence filters it has, likewise
     filter_names: Tuple[str, ...] = ()
+    #: the connections to several residual streams it has, likewise
+    connection_names: Tuple[str, ...] = ()
     needs_mixer = True
     #: True, False, or None for an arrangement that runs with or without a feed-forward
     needs_feed_forward: Optional[bool] = True
 
     def __init__(self, mixer: Optional[Mixer], feed_forward: Optional[FeedForward], norms: Dict[str, Norm],
-                 filters: Optional[Dict[str, "SequenceFilter"]] = None):
+                 filters: Optional[Dict[str, "SequenceFilter"]] = None,
+                 connections: Optional[Dict[str, "Connection"]] = None):
         kind = type(self).__name__
         if (mixer is None) == self.needs_mixer or (self.needs_feed_forward is not None
                                                    and (feed_forward is None) == self.needs_feed_forward):
@@ -242,12 +263,18 @@ class Block:
         if set(filters) != set(self.filter_names):
             raise ValueError(f"{kind}: this arrangement has the filters {sorted(self.filter_names)}, "
                              f"the layer names {sorted(filters)}")
+        connections = dict(connections or {})
+        if set(connections) != set(self.connection_names):
+            raise ValueError(f"{kind}: this arrangement has the connections {sorted(self.connection_names)}, "
+                             f"the layer names {sorted(connections)}")
         self.mixer, self.feed_forward, self.norms, self.filters = mixer, feed_forward, dict(norms), filters
+        self.connections = connections
 
     def parts(self):
         """Every part of the layer by name."""
         out = dict(self.norms)
         out.update(self.filters)
+        out.update(self.connections)
         if self.mixer is not None:
             out["mixer"] = self.mixer
         if self.feed_forward is not None:
@@ -300,7 +327,7 @@ class Runtime:
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
     "norm": {}, "position": {}, "qk_transform": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {},
-    "head": {}, "filter": {},
+    "head": {}, "filter": {}, "connection": {},
 }
 
 
@@ -331,6 +358,10 @@ def register_filter(kind, factory, replace=False):
     _register("filter", kind, factory, replace)
 
 
+def register_connection(kind, factory, replace=False):
+    _register("connection", kind, factory, replace)
+
+
 def register_feed_forward(kind, factory, replace=False):
     _register("feed_forward", kind, factory, replace)
 
@@ -359,12 +390,14 @@ def make_part(family: str, spec) -> Any:
     return reg[spec.kind](**spec.params)
 
 
-def make_block(kind: str, mixer, feed_forward, norms, filters=None) -> Block:
+def make_block(kind: str, mixer, feed_forward, norms, filters=None, connections=None) -> Block:
     """The arrangement ``kind`` around the given parts (``norms``: name -> norm; ``filters``: name ->
-    sequence filter, for an arrangement that has any)."""
+    sequence filter, ``connections``: name -> connection, for an arrangement that has any)."""
     reg = _REGISTRIES["block"]
     if kind not in reg:
         raise ValueError(f"no block arrangement {kind!r}; registered: {sorted(reg)}")
+    if connections:
+        return reg[kind](mixer, feed_forward, norms, filters or {}, connections)
     if filters:
         return reg[kind](mixer, feed_forward, norms, filters)
     return reg[kind](mixer, feed_forward, norms)

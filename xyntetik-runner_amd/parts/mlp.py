@@ -1,9 +1,15 @@
-"""Gated feed-forward: ``down(act(gate(h)) * up(h))``; act = SiLU is the one activation built
-(src/model.c:6399-6407, ``gated_act`` :4451-4452).
+"""Gated feed-forward: ``down(act(gate(h)) * up(h))``; act = SiLU is the one activation the
+products' epilogues apply (src/model.c:6399-6407, ``gated_act`` :4451-4452); "clamped_swish"
+with a limit L shapes both branches (``g' = min(g, L)``, ``u' = clamp(u, -L, L)``,
+``g' sigmoid(1.702 g') (u' + 1)``) and is applied to the product's 32-bit result by a kernel of its own.
 
 ``gate`` and ``up`` are kept as one ``[2F, E]`` matrix so that one product makes both;
 the reference does the reverse for a checkpoint that stores them fused
 (``slice_rows``, src/model.c:238-248).
+
+Routed experts: ``n`` small feed-forwards ``down_e(relu(up_e(h))^2)`` of which every token uses ``top``,
+chosen by a router (32-bit logits, a softmax over all experts, the largest of score + correction;
+the weights are the chosen scores over their sum) and added up with those weights.
 
 Dense feed-forward: ``down(act(up(h)))`` with an activation over the whole row.  "polynorm":
 ``a N(z) + b N(z^2) + c N(z^3) + e`` with four learned numbers, powers element by element and
@@ -22,12 +28,14 @@ class GatedMLP(FeedForward):
     takes_unscaled_rows = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", bias: bool = False,
-                 gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj"):
-        from ..csrc.ops import GATE_ACTIVATIONS
-        if activation not in GATE_ACTIVATIONS:
+                 gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj",
+                 activation_param: float = 0.0, weight_suffix: str = ".weight"):
+        from ..csrc.ops import GATE_ACTIVATIONS, SHAPED_GATES
+        if activation not in GATE_ACTIVATIONS and activation not in SHAPED_GATES:
             raise ValueError(f"gated feed-forward: activation {activation!r} is not built into the kernels "
-                             f"(known: {sorted(GATE_ACTIVATIONS)})")
-        self.activation = activation
+                             f"(known: {sorted(GATE_ACTIVATIONS) + sorted(SHAPED_GATES)})")
+        self.activation, self.activation_param = activation, float(activation_param)
+        self.suffix = weight_suffix
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.bias = bool(bias)
         self.names = (gate_name, up_name, down_name)
@@ -36,8 +44,9 @@ class GatedMLP(FeedForward):
     def param_specs(self) -> Dict[str, ParamSpec]:
         E, F = self.hidden_size, self.intermediate_size
         g, u, d = self.names
-        specs = {f"{g}.weight": ParamSpec((F, E)), f"{u}.weight": ParamSpec((F, E)),
-                 f"{d}.weight": ParamSpec((E, F))}
+        sfx = self.suffix
+        specs = {f"{g}{sfx}": ParamSpec((F, E)), f"{u}{sfx}": ParamSpec((F, E)),
+                 f"{d}{sfx}": ParamSpec((E, F))}
         if self.bias:
             specs.update({f"{g}.bias": ParamSpec((F,), role="vector", init="normal"),
                           f"{u}.bias": ParamSpec((F,), role="vector", init="normal"),
@@ -47,19 +56,27 @@ class GatedMLP(FeedForward):
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         g, u, d = self.names
-        # gate rows then up rows, so that one product makes both; in the kernels' own order
+        sfx = self.suffix
+        from ..csrc.ops import GATE_ACTIVATIONS
+        # gate rows then up rows, so that one product makes both; in the kernels' own order (a gate
+        # that a kernel of its own applies reads the product's plain result)
         self.w_gate_up = rt.ops.pack_weight(
-            torch.cat([tensors[f"{g}.weight"], tensors[f"{u}.weight"]], dim=0).contiguous(), gated=True)
-        self.w_down = rt.ops.pack_weight(tensors[f"{d}.weight"])
+            torch.cat([tensors[f"{g}{sfx}"], tensors[f"{u}{sfx}"]], dim=0).contiguous(),
+            gated=self.activation in GATE_ACTIVATIONS)
+        self.w_down = rt.ops.pack_weight(tensors[f"{d}{sfx}"])
         if self.bias:
             self.b_gate_up = torch.cat([tensors[f"{g}.bias"], tensors[f"{u}.bias"]]).float().contiguous()
             self.b_down = tensors[f"{d}.bias"].float().contiguous()
 
     def _hidden(self, ctx, h):
-        return self.rt.ops.linear_gated(h, self.w_gate_up, bias=self.b_gate_up, activation=self.activation)
+        return self.rt.ops.linear_gated(h, self.w_gate_up, bias=self.b_gate_up, activation=self.activation,
+                                        param=self.activation_param)
 
     def forward(self, ctx, h):
         return self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down)
+
+    def forward_f32(self, ctx, h):
+        return self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down, out_dtype=torch.float32)
 
     def forward_add(self, ctx, h, residual) -> None:
         self.rt.ops.linear(self._hidden(ctx, h), self.w_down, bias=self.b_down, out=residual, accumulate=True)
@@ -108,5 +125,58 @@ class DenseMLP(FeedForward):
         self.rt.ops.linear(self._hidden(ctx, h), self.w_down, out=residual, accumulate=True)
 
 
+class RoutedExperts(FeedForward):
+    """``n`` experts ``down_e(relu(up_e h)^2)`` without biases, ``top`` a token.  Tensors: ``router [n, E]``,
+    ``correction [n]`` (added to the scores for the choice only), and per expert ``e<i>.up [F, E]``,
+    ``e<i>.down [E, F]``.  Nothing here reads the choice on the host: the kernels find a token's
+    experts on the device, so decode steps are recorded like any other."""
+    ACTIVATIONS = ("relu2",)
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, activation: str = "relu2",
+                 router_name: str = "router", correction_name: str = "correction", expert_prefix: str = "e",
+                 up_name: str = "up", down_name: str = "down"):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"routed experts: activation {activation!r} is not built (known: {list(self.ACTIVATIONS)})")
+        if not (1 <= int(top) <= int(num_experts)):
+            raise ValueError(f"routed experts: {top} of {num_experts} experts a token")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.num_experts, self.top = int(num_experts), int(top)
+        self.names = (router_name, correction_name, expert_prefix, up_name, down_name)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E, F = self.hidden_size, self.intermediate_size
+        r, c, p, u, d = self.names
+        # a router of N(0, 0.02) would score all experts alike; a correction that matters is as large as the scores differ
+        specs = {r: ParamSpec((self.num_experts, E), role="vector", init="normal:0.5"),
+                 c: ParamSpec((self.num_experts,), role="vector", init="normal:0.1")}
+        for e in range(self.num_experts):
+            specs[f"{p}{e}.{u}"] = ParamSpec((F, E))
+            specs[f"{p}{e}.{d}"] = ParamSpec((E, F))
+        return specs
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        r, c, p, u, d = self.names
+        self.router = tensors[r].float().contiguous()
+        self.correction = tensors[c].float().contiguous()
+        self.w_up = torch.stack([tensors[f"{p}{e}.{u}"] for e in range(self.num_experts)]).contiguous()
+        self.w_down = torch.stack([tensors[f"{p}{e}.{d}"] for e in range(self.num_experts)]).contiguous()
+
+    def _run(self, ctx, h, out=None, accumulate=False):
+        ops = self.rt.ops
+        idx, wts = ops.moe_route(h, self.router, self.correction, self.top)
+        return ops.moe_experts(h, self.w_up, self.w_down, idx, wts, out=out, accumulate=accumulate)
+
+    def forward(self, ctx, h):
+        return self.rt.ops.convert(self._run(ctx, h), self.rt.dtype)
+
+    def forward_f32(self, ctx, h):
+        return self._run(ctx, h)
+
+    def forward_add(self, ctx, h, residual) -> None:
+        self._run(ctx, h, out=residual, accumulate=True)
+
+
 register_feed_forward("gated_mlp", GatedMLP)
+register_feed_forward("routed_experts", RoutedExperts)
 register_feed_forward("dense_mlp", DenseMLP)

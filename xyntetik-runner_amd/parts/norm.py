@@ -14,15 +14,15 @@ from .base import Norm, ParamSpec, register_norm
 
 
 class RMSNorm(Norm):
-    def __init__(self, size: int, eps: float, weight_name: str = "weight", has_weight: bool = True):
+    def __init__(self, size: int, eps: float, weight_name: str = "weight", has_weight: bool = True, optional: bool = False):
         self.size, self.eps = int(size), float(eps)
-        self.weight_name, self.has_weight = weight_name, has_weight
+        self.weight_name, self.has_weight, self.optional = weight_name, has_weight, bool(optional)
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         if not self.has_weight:
             return {}
-        return {self.weight_name: ParamSpec((self.size,), role="vector", init="ones_jitter")}
+        return {self.weight_name: ParamSpec((self.size,), role="vector", init="ones_jitter", optional=self.optional)}
 
     def bind(self, tensors, rt) -> None:
         self.rt = rt

@@ -5,6 +5,11 @@ in 32-bit floats (``Ops.linear_recurrence``), read out as ``o = S^T q`` after th
 ``q = Wq h``, ``k = Wk h`` (H heads of D), ``v = Wv h`` (H heads of Dv); an optional rotation of the
 first channels of q and k; k times ``D^-1/2`` after it; ``S <- decay_h S + k v^T``.  Every head's
 read-out is divided by its root mean square, then times ``silu(Wg h)``, then ``Wo``.
+Its options make the other members of the family: an activation on q, k and v (``qkv_activation``:
+"silu"), another scale of the keys (``key_scale``; 1 for none), the read-outs of all heads normed
+together instead of head by head (``norm_over``: "row") with a weight a channel (``norm_name``), and
+another gate (``gate_activation``: "sigmoid").  "Lightning attention" is retention with
+``q, k, v = silu(W h)``, no key scale, the joint norm with a weight, and the sigmoid gate.
 
 ``GatedDelta``: the gated delta rule.  ``q``, ``k`` (G heads of D; head h reads head ``h // (H / G)``)
 and ``v`` (H heads of Dv) each pass a short causal convolution over time and SiLU; q and k become
@@ -37,16 +42,28 @@ def _check_sizes(what: str, heads: int, kv_heads: int, dim: int, vdim: int) -> N
 class Retention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, decay: Sequence[float],
                  eps: float, position=None, q_name: str = "q", k_name: str = "k", v_name: str = "v",
-                 g_name: str = "g", o_name: str = "o"):
+                 g_name: str = "g", o_name: str = "o", qkv_activation: Optional[str] = None,
+                 key_scale: Optional[float] = None, norm_over: str = "head", norm_name: Optional[str] = None,
+                 gate_activation: str = "silu"):
         _check_sizes("retention", num_heads, num_heads, head_dim, v_head_dim)
         if len(decay) != num_heads:
             raise ValueError(f"retention: {len(decay)} decays for {num_heads} heads")
+        if qkv_activation not in (None, "silu"):
+            raise ValueError(f"retention: activation {qkv_activation!r} of q, k and v is not built (none, silu)")
+        if norm_over not in ("head", "row"):
+            raise ValueError(f"retention: the read-outs are normed over a 'head' or over the 'row', not {norm_over!r}")
+        if gate_activation not in ("silu", "sigmoid"):
+            raise ValueError(f"retention: gate activation {gate_activation!r} is not built (silu, sigmoid)")
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
         self.head_dim, self.v_head_dim = int(head_dim), int(v_head_dim)
         self.decay_values, self.eps = [float(d) for d in decay], float(eps)
         self.position = make_part("position", position) if position is not None else None
         self.names = (q_name, k_name, v_name, g_name, o_name)
         self.qk_size, self.v_size = self.num_heads * self.head_dim, self.num_heads * self.v_head_dim
+        self.qkv_activation, self.norm_over, self.norm_name = qkv_activation, norm_over, norm_name
+        self.key_scale = float(key_scale) if key_scale is not None else self.head_dim ** -0.5
+        self.gate_activation = gate_activation
+        self.w_norm = None
 
     @property
     def capturable(self) -> bool:
@@ -59,8 +76,12 @@ class Retention(Mixer):
     def param_specs(self) -> Dict[str, ParamSpec]:
         E = self.hidden_size
         q, k, v, g, o = self.names
-        return {q: ParamSpec((self.qk_size, E)), k: ParamSpec((self.qk_size, E)), v: ParamSpec((self.v_size, E)),
-                g: ParamSpec((self.v_size, E)), o: ParamSpec((E, self.v_size))}
+        specs = {q: ParamSpec((self.qk_size, E)), k: ParamSpec((self.qk_size, E)), v: ParamSpec((self.v_size, E)),
+                 g: ParamSpec((self.v_size, E)), o: ParamSpec((E, self.v_size))}
+        if self.norm_name is not None:
+            width = self.v_size if self.norm_over == "row" else self.v_head_dim
+            specs[self.norm_name] = ParamSpec((width,), role="vector", init="ones_jitter")
+        return specs
 
     def bind(self, tensors, rt) -> None:
         self.rt = rt
@@ -68,6 +89,8 @@ class Retention(Mixer):
         self.w_in = rt.ops.pack_weight(torch.cat([tensors[q], tensors[k], tensors[v], tensors[g]], dim=0).contiguous())
         self.w_out = rt.ops.pack_weight(tensors[o])
         self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=rt.device)
+        if self.norm_name is not None:
+            self.w_norm = tensors[self.norm_name].float().contiguous()
         if self.position is not None:
             self.position.bind({}, rt)
             rot = self.position.rotary()
@@ -79,15 +102,23 @@ class Retention(Mixer):
         H, D, Dv, QK, V = self.num_heads, self.head_dim, self.v_head_dim, self.qk_size, self.v_size
         proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         q, k, v, gate = proj[:, :QK], proj[:, QK:2 * QK], proj[:, 2 * QK:2 * QK + V], proj[:, 2 * QK + V:]
+        if self.qkv_activation is not None:
+            ops.act_rows_(proj[:, :2 * QK + V], self.qkv_activation)
         rot = self.position.rotary() if self.position is not None else None
         if rot is not None:
             ops.rotate_rows_(q, ctx.positions, rot.inv_freq, H, D, rot.rotary_dim, 1.0)
-        ops.rotate_rows_(k, ctx.positions, rot.inv_freq if rot else None, H, D, rot.rotary_dim if rot else 0, D ** -0.5)
+        if rot is not None or self.key_scale != 1.0:
+            ops.rotate_rows_(k, ctx.positions, rot.inv_freq if rot else None, H, D, rot.rotary_dim if rot else 0, self.key_scale)
         o = ops.linear_recurrence("retention", q, k, v, cache.state, ctx, H, H, D, Dv, decay=self.decay)
-        return ops.gated_rmsnorm(o, gate, None, H, Dv, self.eps, self.rt.dtype)
+        if self.norm_over == "row":
+            return ops.gated_rmsnorm(o, gate, self.w_norm, 1, V, self.eps, self.rt.dtype, gate_activation=self.gate_activation)
+        return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype, gate_activation=self.gate_activation)
 
     def forward(self, ctx, cache, h):
         return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out)
+
+    def forward_f32(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out_dtype=torch.float32)
 
     def forward_add(self, ctx, cache, h, residual) -> None:
         self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
