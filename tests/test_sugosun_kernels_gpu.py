@@ -116,7 +116,7 @@ def test_streams_write_and_read(ops, S, E):
     close(d.cpu(), new, 3e-6, "write (fused)")
     close(h.float().cpu(), G.rms_norm(u_new, nw, 1e-5), 1e-2, "read after write")
     close(ops.streams_sum(d).cpu(), new.sum(0), 3e-6, "sum")
-    close(ops.streams_expand(dev(y), S).cpu(), np.stack([y] * S), 0, "copies")
+    close(ops.streams_expand(dev(y), S).cpu(), np.stack([y] * S), 1e-7, "copies")
 
 
 # ----------------------------------------------------------------------------- row-wise
@@ -319,7 +319,7 @@ def test_first_tokens_of_a_sequence(tmp_path):
     d = write_random_model(TINY_G1, str(tmp_path / "m"), seed=5, std=0.12, norm_jitter=0.1)
     cfg, w = load_folder(d)
     reqs = {f"r{n}": [int(t) for t in np.random.default_rng(n).integers(0, cfg["vocab"], size=n)] for n in (1, 2, 3, 30)}
-    steps = traces.mixed(reqs, {k: 2 for k in reqs}, max_live=4, seed=1)
+    steps = traces.mixed(reqs, {k: min(2, len(v)) for k, v in reqs.items()}, max_live=4, seed=1)
     from xyntetik_runner_amd.engine.runner import ModelRunner
     from xyntetik_runner_amd.trace import replay
     runner = ModelRunner.from_folder(d, dtype="float32", max_tokens=256, page_size=16, max_requests=4)

@@ -36,27 +36,31 @@ __global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* 
     __syncthreads();
     for (int e = lane; e < n; e += 64) z[e] = expf(z[e] - m) / l;       // the scores
     __syncthreads();
-    // `top` rounds of: the largest score + correction not yet taken, the lower index on a tie
+    // `top` rounds of: the largest score + correction not yet taken, the lower index on a tie.  A score
+    // that is no number (the row of a request that does not exist, whose state is whatever memory held)
+    // counts as the smallest, so that every round still finds an expert that exists.
     float total = 0.f;
-    int mine = -1;          // lane j keeps the j-th choice
+    int mine = 0;           // lane j keeps the j-th choice
     float mine_s = 0.f;
     for (int j = 0; j < top; ++j) {
         float best = -INFINITY;
-        int at = 0x7fffffff;
+        int at = n;         // n: none found yet
         for (int e = lane; e < n; e += 64) {
             const float s = z[e];
-            if (s >= 0.f) {                 // a taken score is stored as -(s) - 1, which is negative
-                const float c = s + correction[e];
-                if (c > best || (c == best && e < at)) { best = c; at = e; }
-            }
+            if (s < -0.5f) continue;        // taken: stored as -(s) - 1
+            float c = s + correction[e];
+            if (!(c == c)) c = -INFINITY;
+            if (at == n || c > best || (c == best && e < at)) { best = c; at = e; }
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
             const float ob = __shfl_xor(best, o, 64);
             const int oa = __shfl_xor(at, o, 64);
-            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+            if (oa < n && (at == n || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
         }
-        const float s = z[at];
+        at = at < n ? at : 0;               // (top <= n: there is always one left; this is for the compiler and for memory that lies)
+        float s = z[at];
+        if (!(s == s) || s < 0.f) s = 0.f;
         total += s;
         if (lane == j) { mine = at; mine_s = s; }
         __syncthreads();
@@ -85,10 +89,10 @@ extern "C" int xr_moe_route(int* idx, float* wts, const void* h, const float* ro
 // z[t * top + j][f] = relu(W_up[e][f] . h[t])^2 for e = idx[t][j].  Grid (T * top, ceil(F / 4)); a wave a column.
 template <typename TW>
 __global__ __launch_bounds__(256) void k_moe_up(TW* __restrict__ z, const TW* __restrict__ h, const TW* __restrict__ w_up,
-                                                const int* __restrict__ idx, int E, int F, int ld_h, int top) {
+                                                const int* __restrict__ idx, int E, int F, int ld_h, int top, int n) {
     const int a = blockIdx.x, f = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (f >= F) return;
-    const int t = a / top, e = idx[a];
+    const int t = a / top, e = min(max(idx[a], 0), n - 1);
     const TW* row = h + (size_t)t * ld_h;
     const TW* w = w_up + ((size_t)e * F + f) * E;
     float acc = 0.f;
@@ -104,12 +108,12 @@ __global__ __launch_bounds__(256) void k_moe_up(TW* __restrict__ z, const TW* __
 template <typename TW>
 __global__ __launch_bounds__(256) void k_moe_down(float* __restrict__ y, const TW* __restrict__ z, const TW* __restrict__ w_down,
                                                   const int* __restrict__ idx, const float* __restrict__ wts, int E, int F,
-                                                  int ld_y, int top, int accumulate) {
+                                                  int ld_y, int top, int n, int accumulate) {
     const int t = blockIdx.x, c = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (c >= E) return;
     float sum = 0.f;
     for (int j = 0; j < top; ++j) {
-        const int e = idx[(size_t)t * top + j];
+        const int e = min(max(idx[(size_t)t * top + j], 0), n - 1);
         const TW* w = w_down + ((size_t)e * E + c) * F;
         const TW* zr = z + ((size_t)t * top + j) * F;
         float acc = 0.f;
@@ -131,11 +135,11 @@ extern "C" int xr_moe_experts(float* y, void* z, const void* h, const void* w_up
     if (T == 0) return XR_OK;
     const dim3 gu(T * top, (F + 3) / 4), gd(T, (E + 3) / 4);
     if (dtype == XR_F32) {
-        k_moe_up<float><<<gu, 256, 0, stream>>>((float*)z, (const float*)h, (const float*)w_up, idx, E, F, ld_h, top);
-        k_moe_down<float><<<gd, 256, 0, stream>>>(y, (const float*)z, (const float*)w_down, idx, wts, E, F, ld_y, top, accumulate);
+        k_moe_up<float><<<gu, 256, 0, stream>>>((float*)z, (const float*)h, (const float*)w_up, idx, E, F, ld_h, top, n);
+        k_moe_down<float><<<gd, 256, 0, stream>>>(y, (const float*)z, (const float*)w_down, idx, wts, E, F, ld_y, top, n, accumulate);
     } else if (dtype == XR_BF16) {
-        k_moe_up<bf16_t><<<gu, 256, 0, stream>>>((bf16_t*)z, (const bf16_t*)h, (const bf16_t*)w_up, idx, E, F, ld_h, top);
-        k_moe_down<bf16_t><<<gd, 256, 0, stream>>>(y, (const bf16_t*)z, (const bf16_t*)w_down, idx, wts, E, F, ld_y, top, accumulate);
+        k_moe_up<bf16_t><<<gu, 256, 0, stream>>>((bf16_t*)z, (const bf16_t*)h, (const bf16_t*)w_up, idx, E, F, ld_h, top, n);
+        k_moe_down<bf16_t><<<gd, 256, 0, stream>>>(y, (const bf16_t*)z, (const bf16_t*)w_down, idx, wts, E, F, ld_y, top, n, accumulate);
     } else { xr_set_error("moe_experts: bad dtype %d", dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("moe_experts");
     return XR_OK;
