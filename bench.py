@@ -307,6 +307,30 @@ def suripel_config(width, layers, vocab=32000):
     return {"architecture": "Suripel", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "layers": out}
 
 
+def sugosun_config(width, layers, vocab=32000):
+    """A Sugosun model of real layer sizes: two residual streams, a pair table of 100,003 rows, heads of 128 in the
+    lightning layers; latent attention with a cached row of 192 + 64 channels, 64 unrotated and 64 rotated query
+    channels a head, values of 128, a query latent of 3/8 width and a window of 1,024; of every four layers
+    lightning with a dense feed-forward of 3.5 x width, latent attention with 16 experts of width / 2 (2 a token),
+    lightning with such experts, latent attention with the dense feed-forward."""
+    H = width // 128
+    dense = {"kind": "dense", "ff": int(width * 3.5), "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 16, "top": 2}}
+    light = {"heads": H, "dim": 128, "vdim": 128, "decay": [1 - 0.06 * 0.75 ** (8 * i / H) for i in range(H)]}
+    latent = {"heads": H, "dim": 64, "rot_dim": 64, "vdim": 128, "q_rank": width * 3 // 8, "kv_rank": 192, "scale": 128 ** -0.5,
+              "rot": {"dims": 64, "base": 1e4}, "mask": {"size": 1024}}
+    out = []
+    for i in range(layers):
+        k = i % 4
+        out.append({"type": "lightning" if k in (0, 2) else "latent_attention", "mixer": light if k in (0, 2) else latent,
+                    "mlp": dense if k in (0, 3) else moe})
+    return {"architecture": "Sugosun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "streams": 2,
+            "embedding": {"bigram": {"buckets": 100003, "mul_prev": 1000003, "mul_cur": 999983}}, "layers": out}
+
+
+DESIGNS = {"suripel": ("Suripel", suripel_config), "sugosun": ("Sugosun", sugosun_config)}
+
+
 def llama_like(width, layers, vocab=32000):
     """The closest existing model at equal size: the Llama decoder with the same width, layers, heads and weights a layer."""
     return dict(LLAMA_3_1_8B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=width // 128,
@@ -353,15 +377,18 @@ def measure_design(runner, vocab, prompt_len, batches, steps, seed):
 
 
 def bench_design(args):
-    """``--design suripel``: prefill and decode of the Suripel design at a few real layer sizes beside the Llama
+    """``--design NAME``: prefill and decode of that design at a few real layer sizes beside the Llama
     decoder of equal size, both with random weights through the same step function.  One JSON line."""
     import torch
+    title, make_config = DESIGNS[args.design]
     sizes = [int(x) for x in args.design_sizes.split(",")]
     batches = [1, 8, 64]
     rows = []
     for width in sizes:
         row = {"width": width, "layers": args.design_layers}
-        for name, cfg in (("suripel", suripel_config(width, args.design_layers)), ("llama", llama_like(width, args.design_layers))):
+        for name, cfg in ((args.design, make_config(width, args.design_layers)), ("llama", llama_like(width, args.design_layers))):
+            if name == "llama" and args.design_alone:
+                continue
             spec, runner = build_runner(cfg, args.dtype, max_tokens=66 * (args.prompt_len + 256), max_requests=64)
             pre, dec = measure_design(runner, 32000, args.prompt_len, batches, min(args.steps, 64), seed=width)
             row[name] = {"prefill_ms": round(pre * 1e3, 3), "prefill_tok_s": round(args.prompt_len / pre, 1),
@@ -371,13 +398,13 @@ def bench_design(args):
             del runner
             torch.cuda.empty_cache()
         rows.append(row)
-    line = {"metric": f"prefill and decode of the Suripel design beside the Llama decoder of equal size ({args.prompt_len}-token prompts, random weights)",
+    line = {"metric": f"prefill and decode of the {title} design beside the Llama decoder of equal size ({args.prompt_len}-token prompts, random weights)",
             "unit": "ms and tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
             "sizes": rows}
     print(json.dumps(line), flush=True)
     if args.record:
         with open(args.record, "w") as f:
-            f.write(f"# bench.py --design suripel\n\nCommand:\n\n    python {' '.join(['bench.py'] + sys.argv[1:])}\n\n"
+            f.write(f"# bench.py --design {args.design}\n\nCommand:\n\n    python {' '.join(['bench.py'] + sys.argv[1:])}\n\n"
                     f"Result (one MI355X, random weights, synthetic tokens):\n\n```json\n{json.dumps(line, indent=1)}\n```\n")
     return 0
 
@@ -404,10 +431,11 @@ def main():
                     help="also write the command and the JSON line into FILE (markdown)")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="also run N requests with prompts of 128..2048 tokens and 128 decoded tokens each through the scheduler")
-    ap.add_argument("--design", default="", choices=["", "suripel"],
+    ap.add_argument("--design", default="", choices=["", "suripel", "sugosun"],
                     help="instead of the serving benchmark: this design at real layer sizes beside the Llama decoder of equal size")
     ap.add_argument("--design-sizes", default="2048,4096", metavar="LIST", help="widths of the --design models")
     ap.add_argument("--design-layers", type=int, default=12, help="layers of the --design models")
+    ap.add_argument("--design-alone", action="store_true", help="the --design model without the Llama decoder beside it")
     args = ap.parse_args()
     if args.design:
         if args.gpus != 1:

@@ -54,7 +54,7 @@ def close(got, want, tol, what=""):
 
 
 # ----------------------------------------------------------------------------- embedding
-@pytest.mark.parametrize("buckets,mp,mc", [(53, 17, 5), (7, 3, 3), (1, 1, 0), (100003, 2147483647, 2147483629), (0, 0, 0)])
+@pytest.mark.parametrize("buckets,mp,mc", [(53, 17, 5), (7, 3, 3), (1, 1, 0), (100003, 2147483647, 2147483629), (1009, 10 ** 15 + 37, 2 ** 40 + 1), (0, 0, 0)])
 def test_pair_hash_embedding_in_portions(ops, buckets, mp, mc):
     """Three requests cut into portions (down to one token), one of them left out of some steps, in
     slots whose last-token entries start as garbage: a portion's first token hashes with the last
@@ -176,6 +176,52 @@ def test_routing(ops, n, top, E):
     assert np.array_equal(idx.cpu().numpy(), chosen), "choice"
     close(wts.cpu(), weights, 5e-6, "weights")
     close(wts.sum(-1).cpu(), np.ones(T), 1e-6, "weights add up to one")
+    # scores that are no numbers (the row of no request) still name experts that exist
+    idx, wts = ops.route_logits(torch.full((3, n), float("nan"), device=DEV), dev(corr), top)
+    assert int(idx.min()) >= 0 and int(idx.max()) < n
+
+
+@pytest.mark.parametrize("T,G,N,K,aw,ow", [(5, 3, 24, 16, 16, 40), (40, 2, 48, 32, 48, 48), (150, 4, 16, 64, 72, 16), (7, 2, 5, 6, 6, 9)])
+def test_products_head_by_head_in_one_launch(ops, T, G, N, K, aw, ow):
+    """Column ranges of wider rows through a matrix a head into column ranges of wider rows; what lies
+    between the ranges stays as it is.  The last case has sizes the matrix cores do not take."""
+    rng = np.random.default_rng(T + G)
+    b16 = lambda x: torch.tensor(x, dtype=torch.float32).to(torch.bfloat16)
+    a = b16(rng.normal(size=(T, (G - 1) * aw + K + 8)))
+    w = b16(rng.normal(size=(G, N, K)) * 0.3)
+    out = torch.full((T, (G - 1) * ow + N + 3), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.heads_linear(a.to(DEV), w.to(DEV), out, G, aw, ow)
+    got = out.float().cpu().numpy()
+    covered = np.zeros(got.shape[1], dtype=bool)
+    for g in range(G):
+        want = a[:, g * aw:g * aw + K].double().numpy() @ w[g].double().numpy().T
+        close(got[:, g * ow:g * ow + N], want, 1e-2, f"head {g}")
+        covered[g * ow:g * ow + N] = True
+    assert (got[:, ~covered] == 7.0).all()
+
+
+@pytest.mark.parametrize("n,top,E,F,T", [(6, 2, 64, 24, 70), (16, 3, 128, 80, 300), (4, 4, 32, 8, 33)])
+def test_experts_over_many_rows_on_the_matrix_cores(ops, n, top, E, F, T):
+    rng = np.random.default_rng(n + T)
+    r16 = (lambda a: torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).to(torch.float64).numpy())
+    h, router, corr = r16(rng.normal(size=(T, E))), r16(rng.normal(size=(n, E)) * 0.4), rng.normal(size=n) * 0.2
+    router[n - 1] = 0.0
+    corr[n - 1] = -100.0                       # an expert that nobody takes (unless every expert is taken)
+    w = {"router": router, "correction": corr}
+    for e in range(n):
+        w[f"e{e}.up"], w[f"e{e}.down"] = r16(rng.normal(size=(F, E)) * 0.3), r16(rng.normal(size=(E, F)) * 0.3)
+    want = G.moe_ff(h, w, n, top)
+    up = dev(np.stack([w[f"e{e}.up"] for e in range(n)]), torch.bfloat16)
+    down = dev(np.stack([w[f"e{e}.down"] for e in range(n)]), torch.bfloat16)
+    assert T * top >= ops.GROUPED_EXPERTS_FROM
+    idx, wts = ops.moe_route(dev(h, torch.bfloat16), dev(router, torch.bfloat16), dev(corr), top)
+    assert np.array_equal(idx.cpu().numpy(), G.route(h, router, corr, top)[0])
+    y = ops.moe_experts(dev(h, torch.bfloat16), up, down, idx, wts)
+    close(y.cpu(), want, 2e-2, "experts, sorted")
+    base = rng.normal(size=(T, E))
+    acc = dev(base)
+    ops.moe_experts(dev(h, torch.bfloat16), up, down, idx, wts, out=acc, accumulate=True)
+    close(acc.cpu(), base + want, 2e-2, "experts added to rows")
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-6), (torch.bfloat16, 2e-2)])
@@ -184,14 +230,14 @@ def test_experts(ops, n, top, E, F, dtype, tol):
     rng = np.random.default_rng(n + E)
     T = 21
     r16 = (lambda a: torch.tensor(a, dtype=torch.float32).to(dtype).to(torch.float64).numpy())
-    h, router, corr = r16(rng.normal(size=(T, E))), rng.normal(size=(n, E)) * 0.4, rng.normal(size=n) * 0.2
+    h, router, corr = r16(rng.normal(size=(T, E))), r16(rng.normal(size=(n, E)) * 0.4), rng.normal(size=n) * 0.2
     w = {"router": router, "correction": corr}
     for e in range(n):
         w[f"e{e}.up"], w[f"e{e}.down"] = r16(rng.normal(size=(F, E)) * 0.3), r16(rng.normal(size=(E, F)) * 0.3)
     want = G.moe_ff(h, w, n, top)
     up = dev(np.stack([w[f"e{e}.up"] for e in range(n)]), dtype)
     down = dev(np.stack([w[f"e{e}.down"] for e in range(n)]), dtype)
-    idx, wts = ops.moe_route(dev(h, dtype), dev(router), dev(corr), top)
+    idx, wts = ops.moe_route(dev(h, dtype), dev(router, dtype), dev(corr), top)
     y = ops.moe_experts(dev(h, dtype), up, down, idx, wts)
     close(y.cpu(), want, tol, "experts")
     base = rng.normal(size=(T, E))

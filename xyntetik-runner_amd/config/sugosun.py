@@ -109,9 +109,10 @@ class SugosunConfig:
         emb = f.mapping("embedding")
         bf = emb.mapping("bigram") if emb is not None else None
         if bf is not None:
-            # the hash is formed in 64-bit integers: token ids below 2^20 times multipliers below 2^31
-            bigram = SugosunBigram(bf.integer("buckets", hi=1 << 30), bf.integer("mul_prev", lo=0, hi=(1 << 31) - 1),
-                                   bf.integer("mul_cur", lo=0, hi=(1 << 31) - 1))
+            # the hash is formed in 64-bit integers from the multipliers' remainders: token ids below 2^20 times
+            # remainders below 2^30
+            bigram = SugosunBigram(bf.integer("buckets", hi=1 << 30), bf.integer("mul_prev", lo=0, hi=1 << 62),
+                                   bf.integer("mul_cur", lo=0, hi=1 << 62))
         loop = None
         lp = f.mapping("loop")
         if lp is not None:

@@ -1,0 +1,250 @@
+// Many small matrix products in one launch, on the matrix cores: out_g = a_g @ w_g^T for groups g
+// that each have a weight matrix [N, K] of their own (bfloat16, 32-bit accumulation).
+//
+//   * heads:   every group has the same T rows; row t of group g is a + t * lda + g * a_group_stride
+//              (a column range of a wider row), its result goes to out + t * ldo + g * o_group_stride.
+//              The per-head products of latent attention (queries into the latent's space, the
+//              attention's output out of it).
+//   * experts: the groups' rows are listed in `perm` (group g owns perm[start .. start + count)),
+//              cut into tiles by k_moe_sort; input row = perm[p] / gather_div, output row = perm[p].
+//              The two products of routed experts over many tokens.
+//
+// A wave computes 16 * RT weight rows x 16 * MT rows with v_mfma_f32_16x16x32_bf16 (weights as the A
+// operand, rows as the B operand: a lane then holds 4 consecutive output columns of one row) and
+// reads its fragments straight from memory, 16 bytes a lane; the four waves of a workgroup take
+// four neighbouring groups of weight rows and share the rows' fragments through the caches.
+// Epilogue: nothing, or relu squared.
+#include "common.h"
+
+typedef __bf16 gm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float gm_f32x4 __attribute__((ext_vector_type(4)));
+
+#define GM_ACT_NONE 0
+#define GM_ACT_RELU2 1
+
+struct GroupedArgs {
+    const bf16_t* a;
+    const bf16_t* w;
+    void* out;
+    long long a_group_stride, w_group_stride, o_group_stride;
+    int lda, ldo, N, K, out_bf16, act;
+    // experts: tiles from the sort; heads: tile_group null, tiles_per_group tiles of every group
+    const int* perm;
+    const int* tile_group;
+    const int* tile_start;
+    const int* tile_count;
+    const int* n_tiles;
+    int gather_div, T, tiles_per_group;
+};
+
+__device__ inline gm_bf16x8 gm_frag(const bf16_t* p, bool ok) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (ok) v = *reinterpret_cast<const uint4*>(p);
+    union { uint4 u; gm_bf16x8 b; } c;
+    c.u = v;
+    return c.b;
+}
+
+template <int MT, int RT>
+__global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs g) {
+    const int tile = blockIdx.x;
+    int group, row0, rows;
+    if (g.tile_group) {
+        if (tile >= *g.n_tiles) return;
+        group = g.tile_group[tile];
+        row0 = g.tile_start[tile];
+        rows = g.tile_count[tile];
+    } else {
+        group = tile / g.tiles_per_group;
+        row0 = (tile - group * g.tiles_per_group) * (16 * MT);
+        rows = g.T - row0 < 16 * MT ? g.T - row0 : 16 * MT;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int n0 = (blockIdx.y * 4 + wave) * (16 * RT);
+    if (n0 >= g.N) return;
+
+    const bf16_t* ap[MT];
+    long long orow[MT];
+    bool a_ok[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int r = i * 16 + l16;
+        a_ok[i] = r < rows;
+        int in_row, out_row;
+        if (g.perm) {
+            const int p = g.perm[row0 + (a_ok[i] ? r : 0)];
+            in_row = p / g.gather_div;
+            out_row = p;
+        } else {
+            in_row = out_row = row0 + (a_ok[i] ? r : 0);
+        }
+        ap[i] = g.a + (long long)in_row * g.lda + (long long)group * g.a_group_stride;
+        orow[i] = (long long)out_row * g.ldo + (long long)group * g.o_group_stride;
+    }
+    const bf16_t* wp[RT];
+    bool w_ok[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        const int n = n0 + r * 16 + l16;
+        w_ok[r] = n < g.N;
+        wp[r] = g.w + (long long)group * g.w_group_stride + (long long)(w_ok[r] ? n : 0) * g.K;
+    }
+    gm_f32x4 acc[RT][MT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[r][i] = gm_f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int k0 = 0; k0 < g.K; k0 += 64) {
+        gm_bf16x8 wf[2][RT], af[2][MT];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k = k0 + u * 32 + lq * 8;
+            const bool k_ok = k < g.K;
+#pragma unroll
+            for (int r = 0; r < RT; ++r) wf[u][r] = gm_frag(wp[r] + k, k_ok && w_ok[r]);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) af[u][i] = gm_frag(ap[i] + k, k_ok && a_ok[i]);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    acc[r][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][r], af[u][i], acc[r][i], 0, 0, 0);
+    }
+    // acc[r][i][e]: output column n0 + r * 16 + 4 * (lane / 16) + e of row i * 16 + lane % 16
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        if (!a_ok[i]) continue;
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const int n = n0 + r * 16 + lq * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (n + e >= g.N) continue;
+                float v = acc[r][i][e];
+                if (g.act == GM_ACT_RELU2) { v = fmaxf(v, 0.f); v *= v; }
+                if (g.out_bf16) ((bf16_t*)g.out)[orow[i] + n + e] = f32_to_bf16(v);
+                else ((float*)g.out)[orow[i] + n + e] = v;
+            }
+        }
+    }
+}
+
+static int launch_grouped(const GroupedArgs& g, int n_tiles_max, int rows_a_tile, hipStream_t stream) {
+    const dim3 grid(n_tiles_max, (g.N + 127) / 128);       // 4 waves x 2 groups of 16 weight rows
+    if (rows_a_tile == 16) k_grouped_gemm<1, 2><<<grid, 256, 0, stream>>>(g);
+    else if (rows_a_tile == 32) k_grouped_gemm<2, 2><<<grid, 256, 0, stream>>>(g);
+    else k_grouped_gemm<4, 2><<<grid, 256, 0, stream>>>(g);
+    return 0;
+}
+
+static bool grouped_operands_ok(const void* a, const void* w, int K, int lda, long long a_gs, long long w_gs) {
+    return K % 8 == 0 && lda % 8 == 0 && a_gs % 8 == 0 && w_gs % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0;
+}
+
+// out[t][g][:N] = w[g] @ a[t][g][:K] for G groups and T rows; a, out: column ranges of wider rows.
+extern "C" int xr_heads_gemm_bf16(void* out, const void* a, const void* w, int T, int G, int N, int K, int lda,
+                                  long long a_group_stride, int ldo, long long o_group_stride, int out_dtype, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && G > 0 && N > 0 && K > 0, "heads_gemm: bad sizes T=%d G=%d N=%d K=%d", T, G, N, K);
+    XR_REQUIRE(out_dtype == XR_F32 || out_dtype == XR_BF16, "heads_gemm: bad output dtype %d", out_dtype);
+    XR_REQUIRE(grouped_operands_ok(a, w, K, lda, a_group_stride, (long long)N * K),
+               "heads_gemm: K, the row stride and the groups' offsets must be multiples of 8 and the operands 16-byte aligned");
+    if (T == 0) return XR_OK;
+    const int bm = T <= 16 ? 16 : (T <= 32 ? 32 : 64);
+    GroupedArgs g{};
+    g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.out = out;
+    g.a_group_stride = a_group_stride; g.w_group_stride = (long long)N * K; g.o_group_stride = o_group_stride;
+    g.lda = lda; g.ldo = ldo; g.N = N; g.K = K; g.out_bf16 = out_dtype == XR_BF16; g.act = GM_ACT_NONE;
+    g.gather_div = 1; g.T = T; g.tiles_per_group = (T + bm - 1) / bm;
+    XR_REQUIRE((long long)G * g.tiles_per_group <= 0x7fffffffLL, "heads_gemm: too many tiles");
+    launch_grouped(g, G * g.tiles_per_group, bm, stream);
+    XR_CHECK_LAUNCH("heads_gemm");
+    return XR_OK;
+}
+
+// ---------------------------------------------------------------- the experts' rows, sorted by expert
+// A = T * top choices idx[a] (a = token * top + j).  One workgroup: counts, offsets, the list `perm` of
+// the choices expert by expert (in any order inside an expert: a row's result does not depend on
+// its place), and the tiles of `bm` rows: tile_group / tile_start / tile_count, n_tiles[0] of them.
+#define SORT_MAX_EXPERTS 1024
+__global__ __launch_bounds__(1024) void k_moe_sort(const int* __restrict__ idx, int A, int n, int bm, int* __restrict__ perm,
+                                                    int* __restrict__ tile_group, int* __restrict__ tile_start,
+                                                    int* __restrict__ tile_count, int* __restrict__ n_tiles) {
+    __shared__ int count[SORT_MAX_EXPERTS], offset[SORT_MAX_EXPERTS], cursor[SORT_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < n; e += 1024) { count[e] = 0; cursor[e] = 0; }
+    __syncthreads();
+    for (int a = threadIdx.x; a < A; a += 1024) atomicAdd(&count[min(max(idx[a], 0), n - 1)], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, t = 0;
+        for (int e = 0; e < n; ++e) {
+            offset[e] = at;
+            for (int s = 0; s < count[e]; s += bm) {
+                tile_group[t] = e;
+                tile_start[t] = at + s;
+                tile_count[t] = count[e] - s < bm ? count[e] - s : bm;
+                ++t;
+            }
+            at += count[e];
+        }
+        n_tiles[0] = t;
+    }
+    __syncthreads();
+    for (int a = threadIdx.x; a < A; a += 1024) {
+        const int e = min(max(idx[a], 0), n - 1);
+        perm[offset[e] + atomicAdd(&cursor[e], 1)] = a;
+    }
+}
+
+// y[t] (+)= sum_j wts[t][j] * yz[t * top + j], in the order of the choice
+__global__ void k_moe_combine(float* __restrict__ y, const float* __restrict__ yz, const float* __restrict__ wts, int E, int ld_y,
+                              int top, size_t n, int accumulate) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / E;
+    const int c = (int)(i - t * E);
+    float s = 0.f;
+    for (int j = 0; j < top; ++j) s += wts[t * top + j] * yz[(t * top + j) * E + c];
+    float* o = y + t * ld_y + c;
+    *o = accumulate ? *o + s : s;
+}
+
+// The routed experts over many rows: sort, z = relu(up)^2 by expert, yz = down by expert, y = the weighted sum.
+// scratch: ints [A + 3 * max_tiles + 1]; z: bf16 [A, F]; yz: float [A, E].  max_tiles = ceil(A / 64) + n.
+extern "C" int xr_moe_experts_grouped(float* y, void* z, float* yz, int* scratch, const void* h, const void* w_up,
+                                      const void* w_down, const int* idx, const float* wts, int T, int E, int F, int ld_h,
+                                      int ld_y, int n, int top, int accumulate, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && E > 0 && F > 0 && ld_h >= E && ld_y >= E, "moe_experts_grouped: bad sizes T=%d E=%d F=%d", T, E, F);
+    XR_REQUIRE(n >= 1 && n <= SORT_MAX_EXPERTS && top >= 1 && top <= n, "moe_experts_grouped: %d experts (at most %d), %d chosen", n,
+               SORT_MAX_EXPERTS, top);
+    XR_REQUIRE((long long)T * top <= (1 << 24), "moe_experts_grouped: too many rows");
+    XR_REQUIRE(grouped_operands_ok(h, w_up, E, ld_h, 0, (long long)F * E) && grouped_operands_ok(z, w_down, F, F, 0, (long long)E * F),
+               "moe_experts_grouped: widths and row strides must be multiples of 8 and the operands 16-byte aligned");
+    if (T == 0) return XR_OK;
+    const int A = T * top, bm = 64, max_tiles = (A + bm - 1) / bm + n;
+    int* perm = scratch;
+    int* tile_group = perm + A;
+    int* tile_start = tile_group + max_tiles;
+    int* tile_count = tile_start + max_tiles;
+    int* n_tiles = tile_count + max_tiles;
+    k_moe_sort<<<1, 1024, 0, stream>>>(idx, A, n, bm, perm, tile_group, tile_start, tile_count, n_tiles);
+    GroupedArgs g{};
+    g.perm = perm; g.tile_group = tile_group; g.tile_start = tile_start; g.tile_count = tile_count; g.n_tiles = n_tiles;
+    g.a_group_stride = 0; g.o_group_stride = 0;
+    // up: rows of h by token, results by choice
+    g.a = (const bf16_t*)h; g.lda = ld_h; g.w = (const bf16_t*)w_up; g.w_group_stride = (long long)F * E; g.out = z; g.ldo = F;
+    g.N = F; g.K = E; g.out_bf16 = 1; g.act = GM_ACT_RELU2; g.gather_div = top;
+    launch_grouped(g, max_tiles, bm, stream);
+    // down: rows of z by choice, results by choice
+    g.a = (const bf16_t*)z; g.lda = F; g.w = (const bf16_t*)w_down; g.w_group_stride = (long long)E * F; g.out = yz; g.ldo = E;
+    g.N = E; g.K = F; g.out_bf16 = 0; g.act = GM_ACT_NONE; g.gather_div = 1;
+    launch_grouped(g, max_tiles, bm, stream);
+    const size_t cnt = (size_t)T * E;
+    k_moe_combine<<<(unsigned)((cnt + 255) / 256), 256, 0, stream>>>(y, yz, wts, E, ld_y, top, cnt, accumulate);
+    XR_CHECK_LAUNCH("moe_experts_grouped");
+    return XR_OK;
+}

@@ -1,8 +1,8 @@
 // A feed-forward of many small experts of which every token uses a few ("mixture of experts").
 //
-// k_moe_route: per token the router's logits in 32 bits, a softmax over all experts, the `top`
-// experts with the largest score + correction (ties: the lower index), and their weights: the
-// chosen scores (without the correction) over their sum + 1e-20.
+// k_moe_route: per token, from the router's 32-bit logits (a matrix product of its own), a softmax over
+// all experts, the `top` experts with the largest score + correction (ties: the lower index), and
+// their weights: the chosen scores (without the correction) over their sum + 1e-20.
 // k_moe_up / k_moe_down: the experts' two products token by token, a wave an output column, the
 // weights of the chosen experts streamed: what a few decoded tokens need.  Expert:
 // down(act(up h)), act = relu squared.  The down product adds a token's experts up in the order
@@ -12,20 +12,11 @@
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOP 16
 
-template <typename TH>
-__global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* __restrict__ wts, const TH* __restrict__ h,
-                                                  const float* __restrict__ router, const float* __restrict__ correction,
-                                                  int E, int ld_h, int n, int top) {
+__global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ logits,
+                                                  const float* __restrict__ correction, int ld, int n, int top) {
     __shared__ float z[MOE_MAX_EXPERTS];
     const int t = blockIdx.x, lane = threadIdx.x;
-    const TH* row = h + (size_t)t * ld_h;
-    for (int e = 0; e < n; ++e) {
-        const float* w = router + (size_t)e * E;
-        float a = 0.f;
-        for (int i = lane; i < E; i += 64) a += ld<TH>(row, i) * w[i];
-        a = wave_sum(a);
-        if (lane == 0) z[e] = a;
-    }
+    for (int e = lane; e < n; e += 64) z[e] = logits[(size_t)t * ld + e];
     __syncthreads();
     float m = -INFINITY;
     for (int e = lane; e < n; e += 64) m = fmaxf(m, z[e]);
@@ -73,31 +64,60 @@ __global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* 
     }
 }
 
-extern "C" int xr_moe_route(int* idx, float* wts, const void* h, const float* router, const float* correction, int T, int E,
-                            int ld_h, int n, int top, int h_dtype, hipStream_t stream) {
-    XR_REQUIRE(T >= 0 && E > 0 && ld_h >= E, "moe_route: bad sizes T=%d E=%d ld=%d", T, E, ld_h);
+extern "C" int xr_moe_route(int* idx, float* wts, const float* logits, const float* correction, int T, int ld, int n, int top,
+                            hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && ld >= n, "moe_route: bad sizes T=%d ld=%d", T, ld);
     XR_REQUIRE(n >= 1 && n <= MOE_MAX_EXPERTS && top >= 1 && top <= n && top <= MOE_MAX_TOP,
                "moe_route: %d experts (at most %d), %d chosen (at most %d)", n, MOE_MAX_EXPERTS, top, MOE_MAX_TOP);
     if (T == 0) return XR_OK;
-    if (h_dtype == XR_F32) k_moe_route<float><<<T, 64, 0, stream>>>(idx, wts, (const float*)h, router, correction, E, ld_h, n, top);
-    else if (h_dtype == XR_BF16) k_moe_route<bf16_t><<<T, 64, 0, stream>>>(idx, wts, (const bf16_t*)h, router, correction, E, ld_h, n, top);
-    else { xr_set_error("moe_route: bad dtype %d", h_dtype); return XR_BAD_ARG; }
+    k_moe_route<<<T, 64, 0, stream>>>(idx, wts, logits, correction, ld, n, top);
     XR_CHECK_LAUNCH("moe_route");
     return XR_OK;
+}
+
+// A wave's dot product of two rows of n elements; `vec`: both rows start on 16 bytes and n is a multiple of
+// 8 (bfloat16) or 4 (float), so a lane reads 16 bytes at a time.
+template <typename TW> __device__ inline float wave_dot(const TW* __restrict__ w, const TW* __restrict__ x, int n, int lane, bool vec);
+template <> __device__ inline float wave_dot<float>(const float* __restrict__ w, const float* __restrict__ x, int n, int lane, bool vec) {
+    float acc = 0.f;
+    if (vec) {
+        for (int i = lane * 4; i < n; i += 256) {
+            const float4 a = *reinterpret_cast<const float4*>(w + i), b = *reinterpret_cast<const float4*>(x + i);
+            acc = fmaf(a.x, b.x, acc); acc = fmaf(a.y, b.y, acc); acc = fmaf(a.z, b.z, acc); acc = fmaf(a.w, b.w, acc);
+        }
+    } else {
+        for (int i = lane; i < n; i += 64) acc = fmaf(w[i], x[i], acc);
+    }
+    return wave_sum(acc);
+}
+__device__ inline float bf_lo(uint32_t v) { return __uint_as_float(v << 16); }
+__device__ inline float bf_hi(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+template <> __device__ inline float wave_dot<bf16_t>(const bf16_t* __restrict__ w, const bf16_t* __restrict__ x, int n, int lane, bool vec) {
+    float acc = 0.f;
+    if (vec) {
+        for (int i = lane * 8; i < n; i += 512) {
+            const uint4 a = *reinterpret_cast<const uint4*>(w + i), b = *reinterpret_cast<const uint4*>(x + i);
+            acc = fmaf(bf_lo(a.x), bf_lo(b.x), acc); acc = fmaf(bf_hi(a.x), bf_hi(b.x), acc);
+            acc = fmaf(bf_lo(a.y), bf_lo(b.y), acc); acc = fmaf(bf_hi(a.y), bf_hi(b.y), acc);
+            acc = fmaf(bf_lo(a.z), bf_lo(b.z), acc); acc = fmaf(bf_hi(a.z), bf_hi(b.z), acc);
+            acc = fmaf(bf_lo(a.w), bf_lo(b.w), acc); acc = fmaf(bf_hi(a.w), bf_hi(b.w), acc);
+        }
+    } else {
+        for (int i = lane; i < n; i += 64) acc = fmaf(bf16_to_f32(w[i]), bf16_to_f32(x[i]), acc);
+    }
+    return wave_sum(acc);
 }
 
 // z[t * top + j][f] = relu(W_up[e][f] . h[t])^2 for e = idx[t][j].  Grid (T * top, ceil(F / 4)); a wave a column.
 template <typename TW>
 __global__ __launch_bounds__(256) void k_moe_up(TW* __restrict__ z, const TW* __restrict__ h, const TW* __restrict__ w_up,
-                                                const int* __restrict__ idx, int E, int F, int ld_h, int top, int n) {
+                                                const int* __restrict__ idx, int E, int F, int ld_h, int top, int n, int vec) {
     const int a = blockIdx.x, f = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (f >= F) return;
     const int t = a / top, e = min(max(idx[a], 0), n - 1);
     const TW* row = h + (size_t)t * ld_h;
     const TW* w = w_up + ((size_t)e * F + f) * E;
-    float acc = 0.f;
-    for (int i = lane; i < E; i += 64) acc += ld<TW>(w, i) * ld<TW>(row, i);
-    acc = wave_sum(acc);
+    const float acc = wave_dot<TW>(w, row, E, lane, vec != 0);
     if (lane == 0) {
         const float r = fmaxf(acc, 0.f);
         st<TW>(z, (size_t)a * F + f, r * r);
@@ -108,7 +128,7 @@ __global__ __launch_bounds__(256) void k_moe_up(TW* __restrict__ z, const TW* __
 template <typename TW>
 __global__ __launch_bounds__(256) void k_moe_down(float* __restrict__ y, const TW* __restrict__ z, const TW* __restrict__ w_down,
                                                   const int* __restrict__ idx, const float* __restrict__ wts, int E, int F,
-                                                  int ld_y, int top, int n, int accumulate) {
+                                                  int ld_y, int top, int n, int accumulate, int vec) {
     const int t = blockIdx.x, c = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (c >= E) return;
     float sum = 0.f;
@@ -116,9 +136,7 @@ __global__ __launch_bounds__(256) void k_moe_down(float* __restrict__ y, const T
         const int e = min(max(idx[(size_t)t * top + j], 0), n - 1);
         const TW* w = w_down + ((size_t)e * E + c) * F;
         const TW* zr = z + ((size_t)t * top + j) * F;
-        float acc = 0.f;
-        for (int i = lane; i < F; i += 64) acc += ld<TW>(w, i) * ld<TW>(zr, i);
-        sum += wts[(size_t)t * top + j] * wave_sum(acc);
+        sum += wts[(size_t)t * top + j] * wave_dot<TW>(w, zr, F, lane, vec != 0);
     }
     if (lane == 0) {
         float* o = y + (size_t)t * ld_y + c;
@@ -134,12 +152,15 @@ extern "C" int xr_moe_experts(float* y, void* z, const void* h, const void* w_up
     XR_REQUIRE((long long)T * top <= 0x7fffffffLL, "moe_experts: too many rows");
     if (T == 0) return XR_OK;
     const dim3 gu(T * top, (F + 3) / 4), gd(T, (E + 3) / 4);
+    const int per16 = dtype == XR_BF16 ? 8 : 4;             // elements in 16 bytes
+    const bool al = ((uintptr_t)h % 16) == 0 && ((uintptr_t)w_up % 16) == 0 && ((uintptr_t)w_down % 16) == 0 && ((uintptr_t)z % 16) == 0;
+    const int vu = al && E % per16 == 0 && ld_h % per16 == 0, vd = al && F % per16 == 0;
     if (dtype == XR_F32) {
-        k_moe_up<float><<<gu, 256, 0, stream>>>((float*)z, (const float*)h, (const float*)w_up, idx, E, F, ld_h, top, n);
-        k_moe_down<float><<<gd, 256, 0, stream>>>(y, (const float*)z, (const float*)w_down, idx, wts, E, F, ld_y, top, n, accumulate);
+        k_moe_up<float><<<gu, 256, 0, stream>>>((float*)z, (const float*)h, (const float*)w_up, idx, E, F, ld_h, top, n, vu);
+        k_moe_down<float><<<gd, 256, 0, stream>>>(y, (const float*)z, (const float*)w_down, idx, wts, E, F, ld_y, top, n, accumulate, vd);
     } else if (dtype == XR_BF16) {
-        k_moe_up<bf16_t><<<gu, 256, 0, stream>>>((bf16_t*)z, (const bf16_t*)h, (const bf16_t*)w_up, idx, E, F, ld_h, top, n);
-        k_moe_down<bf16_t><<<gd, 256, 0, stream>>>(y, (const bf16_t*)z, (const bf16_t*)w_down, idx, wts, E, F, ld_y, top, n, accumulate);
+        k_moe_up<bf16_t><<<gu, 256, 0, stream>>>((bf16_t*)z, (const bf16_t*)h, (const bf16_t*)w_up, idx, E, F, ld_h, top, n, vu);
+        k_moe_down<bf16_t><<<gd, 256, 0, stream>>>(y, (const bf16_t*)z, (const bf16_t*)w_down, idx, wts, E, F, ld_y, top, n, accumulate, vd);
     } else { xr_set_error("moe_experts: bad dtype %d", dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("moe_experts");
     return XR_OK;

@@ -74,7 +74,9 @@ _PROTOS = {
     "xr_streams_sum": [_p, _p, _i, _i, _i, _p],
     "xr_streams_step": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
     "xr_latent_prepare": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p],
-    "xr_moe_route": [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p],
+    "xr_moe_route": [_p, _p, _p, _p, _i, _i, _i, _i, _p],
+    "xr_moe_experts_grouped": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_heads_gemm_bf16": [_p, _p, _p, _i, _i, _i, _i, _i, C.c_longlong, _i, C.c_longlong, _i, _p],
     "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
     "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p],
@@ -778,6 +780,8 @@ class Ops:
                 raise KernelError("embedding_pairs: the requests' last tokens must be int32 [slots]")
         if norm_w is not None and (norm_w.dtype != torch.float32 or norm_w.numel() != E or not norm_w.is_contiguous()):
             raise KernelError(f"embedding_pairs: the norm's weight must be float32 [{E}]")
+        if buckets:     # (a b) mod n = ((a mod n)(b mod n)) mod n: the kernel's 64-bit products then hold any multiplier
+            mul_prev, mul_cur = int(mul_prev) % int(buckets), int(mul_cur) % int(buckets)
         T = ids.numel()
         out = torch.empty((T, E), dtype=torch.float32, device=table.device)
         self.lib.check(self.lib.xr_embedding_pairs(out.data_ptr(), table.data_ptr(), _ptr(pairs), _ptr(norm_w), ids.data_ptr(),
@@ -876,24 +880,51 @@ class Ops:
                                                   float(eps), dtype_code(dt), _stream()))
         return qn
 
+    def heads_linear(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, G: int, a_width: int, out_width: int) -> None:
+        """``out[:, g * out_width : g * out_width + N] = a[:, g * a_width : g * a_width + K] @ w[g]^T`` for the ``G``
+        groups (heads) of ``w [G, N, K]``: every head's column range of the rows ``a`` through a matrix of the
+        head's own, into the head's column range of ``out``.  bfloat16 with sizes the matrix cores take
+        (``K`` and the ranges' starts multiples of 8) runs as one launch; everything else head by head."""
+        self._dev(a, w, out)
+        T = a.shape[0]
+        Gw, N, K = w.shape
+        if Gw != G or a.stride(1) != 1 or out.stride(1) != 1 or a.shape[1] < (G - 1) * a_width + K or out.shape[1] < (G - 1) * out_width + N:
+            raise KernelError("heads_linear: the heads' column ranges do not fit the rows")
+        if a.dtype != w.dtype:
+            raise KernelError(f"heads_linear: rows are {a.dtype}, weights {w.dtype}")
+        self._contig(w, "heads_linear weights")
+        if (self.use_mfma and a.dtype == torch.bfloat16 and K % 8 == 0 and a_width % 8 == 0 and a.stride(0) % 8 == 0
+                and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and (N * K) % 8 == 0):
+            self.lib.check(self.lib.xr_heads_gemm_bf16(out.data_ptr(), a.data_ptr(), w.data_ptr(), T, G, N, K, a.stride(0),
+                                                       a_width, out.stride(0), out_width, dtype_code(out.dtype), _stream()))
+            return
+        for g in range(G):
+            self.linear(a[:, g * a_width:g * a_width + K], w[g], out=out[:, g * out_width:g * out_width + N])
+
     # -- mixture of experts ------------------------------------------------------------
-    def moe_route(self, h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int):
-        """``(experts [T, top] int32, weights [T, top] float32)``: 32-bit logits ``router [n, E] @ h``, a softmax
-        over all experts, the ``top`` largest of score + ``correction`` (the lower index on a tie), weights =
-        the chosen scores over their sum + 1e-20."""
-        self._dev(h, router, correction)
-        if h.dim() != 2 or h.stride(1) != 1:
-            raise KernelError("moe_route: h must be [rows, width] with unit column stride")
-        T, E = h.shape
-        n = router.shape[0]
-        if (router.dtype != torch.float32 or tuple(router.shape) != (n, E) or not router.is_contiguous()
-                or correction.dtype != torch.float32 or correction.numel() != n):
-            raise KernelError(f"moe_route: router must be float32 [{n}, {E}] and the correction float32 [{n}]")
-        idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
-        wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
-        self.lib.check(self.lib.xr_moe_route(idx.data_ptr(), wts.data_ptr(), h.data_ptr(), router.data_ptr(), correction.data_ptr(),
-                                             T, E, h.stride(0), n, int(top), dtype_code(h.dtype), _stream()))
+    def moe_route(self, h: torch.Tensor, router, correction: torch.Tensor, top: int):
+        """``(experts [T, top] int32, weights [T, top] float32)``: 32-bit logits ``h @ router [n, E]^T`` (a matrix
+        product with 32-bit accumulation and a 32-bit result; ``router`` in ``h``'s dtype, a matrix or a
+        ``PackedWeight``), a softmax over all experts, the ``top`` largest of score + ``correction`` (the lower
+        index on a tie), weights = the chosen scores over their sum + 1e-20."""
+        logits = self.linear(h, router, out_dtype=torch.float32)
+        return self.route_logits(logits, correction, top)
+
+    def route_logits(self, logits: torch.Tensor, correction: torch.Tensor, top: int):
+        """``moe_route`` from the 32-bit logits ``[T, n]``."""
+        self._dev(logits, correction)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise KernelError("route_logits: logits must be float32 [rows, experts] with unit column stride")
+        T, n = logits.shape
+        if correction.dtype != torch.float32 or correction.numel() != n:
+            raise KernelError(f"route_logits: the correction must be float32 [{n}]")
+        idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        wts = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+        self.lib.check(self.lib.xr_moe_route(idx.data_ptr(), wts.data_ptr(), logits.data_ptr(), correction.data_ptr(), T,
+                                             logits.stride(0), n, int(top), _stream()))
         return idx, wts
+
+    GROUPED_EXPERTS_FROM = 32       # choices (rows x top) from which the experts' rows are sorted and run on the matrix cores
 
     def moe_experts(self, h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor,
                     out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
@@ -916,6 +947,17 @@ class Ops:
         elif out.dtype != torch.float32 or tuple(out.shape) != (T, E) or out.stride(1) != 1:
             raise KernelError(f"moe_experts: the output must be float32 [{T}, {E}]")
         z = torch.empty((T * top, F), dtype=h.dtype, device=h.device)
+        if (self.use_mfma and h.dtype == torch.bfloat16 and T * top >= self.GROUPED_EXPERTS_FROM and E % 8 == 0 and F % 8 == 0
+                and h.stride(0) % 8 == 0 and h.data_ptr() % 16 == 0 and n <= 1024 and T * top <= (1 << 24)):
+            # many rows: sorted by expert, both products on the matrix cores, then the weighted sum
+            A = T * top
+            yz = torch.empty((A, E), dtype=torch.float32, device=h.device)
+            scratch = torch.empty((A + 3 * (-(-A // 64) + n) + 1,), dtype=torch.int32, device=h.device)
+            self.lib.check(self.lib.xr_moe_experts_grouped(out.data_ptr(), z.data_ptr(), yz.data_ptr(), scratch.data_ptr(),
+                                                           h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(),
+                                                           wts.data_ptr(), T, E, F, h.stride(0), out.stride(0), n, top,
+                                                           1 if accumulate else 0, _stream()))
+            return out
         self.lib.check(self.lib.xr_moe_experts(out.data_ptr(), z.data_ptr(), h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(),
                                                idx.data_ptr(), wts.data_ptr(), T, E, F, h.stride(0), out.stride(0), n, top,
                                                1 if accumulate else 0, dtype_code(h.dtype), _stream()))

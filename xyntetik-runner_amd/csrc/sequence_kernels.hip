@@ -362,12 +362,39 @@ __global__ __launch_bounds__(64) void k_gated_rmsnorm(TO* __restrict__ out, cons
     }
 }
 
+// The same with a workgroup of 256 a (token, head), for long rows (all heads normed together).
+template <typename TO>
+__global__ __launch_bounds__(256) void k_gated_rmsnorm_wide(TO* __restrict__ out, const float* __restrict__ o,
+                                                           const float* __restrict__ gate, const float* __restrict__ w,
+                                                           int H, int Dv, int ld_g, float eps, int w_full, int gate_act) {
+    __shared__ float part[4];
+    const int t = blockIdx.x, h = blockIdx.y;
+    const float* orow = o + ((size_t)t * H + h) * Dv;
+    const float* grow = gate + (size_t)t * ld_g + (size_t)h * Dv;
+    const float* wrow = w ? (w_full ? w + (size_t)h * Dv : w) : nullptr;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < Dv; d += 256) ss += orow[d] * orow[d];
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float rinv = 1.0f / sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)Dv + eps);
+    TO* dst = out + ((size_t)t * H + h) * Dv;
+    for (int d = threadIdx.x; d < Dv; d += 256) {
+        const float g = grow[d];
+        const float sg = 1.0f / (1.0f + expf(-g));
+        st<TO>(dst, d, orow[d] * rinv * (wrow ? wrow[d] : 1.f) * (gate_act == XR_GATE_SIGMOID ? sg : g * sg));
+    }
+}
+
 extern "C" int xr_gated_rmsnorm(void* out, const float* o, const float* gate, const float* w, int T, int H, int Dv,
                                 int ld_g, float eps, int out_dtype, int w_full, int gate_act, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && H > 0 && Dv > 0 && ld_g >= H * Dv, "gated_rmsnorm: bad sizes T=%d H=%d Dv=%d ld=%d", T, H, Dv, ld_g);
     XR_REQUIRE(gate_act == XR_GATE_SILU || gate_act == XR_GATE_SIGMOID, "gated_rmsnorm: unknown gate activation %d", gate_act);
     if (T == 0) return XR_OK;
-    if (out_dtype == XR_F32) k_gated_rmsnorm<float><<<dim3(T, H), 64, 0, stream>>>((float*)out, o, gate, w, H, Dv, ld_g, eps, w_full, gate_act);
+    const bool wide = Dv > 256;       // (the sums' order differs between the two kernels, not between calls of one size)
+    if (out_dtype == XR_F32 && wide) k_gated_rmsnorm_wide<float><<<dim3(T, H), 256, 0, stream>>>((float*)out, o, gate, w, H, Dv, ld_g, eps, w_full, gate_act);
+    else if (out_dtype == XR_BF16 && wide) k_gated_rmsnorm_wide<bf16_t><<<dim3(T, H), 256, 0, stream>>>((bf16_t*)out, o, gate, w, H, Dv, ld_g, eps, w_full, gate_act);
+    else if (out_dtype == XR_F32) k_gated_rmsnorm<float><<<dim3(T, H), 64, 0, stream>>>((float*)out, o, gate, w, H, Dv, ld_g, eps, w_full, gate_act);
     else if (out_dtype == XR_BF16) k_gated_rmsnorm<bf16_t><<<dim3(T, H), 64, 0, stream>>>((bf16_t*)out, o, gate, w, H, Dv, ld_g, eps, w_full, gate_act);
     else { xr_set_error("gated_rmsnorm: bad dtype %d", out_dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("gated_rmsnorm");

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void k_embedding_pairs(float* __restrict__ out
     if (pairs) {
         long long r = buckets;
         if (positions[t] != 0) {
-            r = ((long long)s_prev * mul_prev + (long long)id * mul_cur) % (long long)buckets;
+            r = (((long long)s_prev % buckets) * mul_prev + ((long long)id % buckets) * mul_cur) % (long long)buckets;
             if (r < 0) r += buckets;
         }
         prow = pairs + (size_t)r * E;
@@ -179,6 +179,107 @@ __global__ __launch_bounds__(256) void k_streams_step(float* __restrict__ xs, co
     }
 }
 
+// The same for rows whose width is a multiple of 4 (up to 4 * 256 * NV): a thread handles float4 pieces,
+// and keeps u in registers between the sum and the scaling.
+template <typename TO> __device__ inline void hc_store4(TO* p, size_t i, float a, float b, float c, float d);
+template <> __device__ inline void hc_store4<float>(float* p, size_t i, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(p + i) = make_float4(a, b, c, d);
+}
+template <> __device__ inline void hc_store4<bf16_t>(bf16_t* p, size_t i, float a, float b, float c, float d) {
+    uint2 w;
+    w.x = pack_bf16x2(a, b);
+    w.y = pack_bf16x2(c, d);
+    *reinterpret_cast<uint2*>(p + i) = w;
+}
+
+template <typename TO, int NV>
+__global__ __launch_bounds__(256) void k_streams_step_v4(float* __restrict__ xs, const float* __restrict__ y,
+                                                         const float* __restrict__ mix, const float* __restrict__ out_w,
+                                                         const float* __restrict__ in_w, const float* __restrict__ norm_w,
+                                                         TO* __restrict__ h, int T, int E, int S, float eps) {
+    __shared__ float part[4];
+    __shared__ float c_mix[HC_MAX_STREAMS * HC_MAX_STREAMS], c_out[HC_MAX_STREAMS], c_in[HC_MAX_STREAMS];
+    const int t = blockIdx.x;
+    if (threadIdx.x < S * S && y) c_mix[threadIdx.x] = mix[threadIdx.x];
+    if (threadIdx.x < S) {
+        if (y) c_out[threadIdx.x] = out_w[threadIdx.x];
+        if (h) c_in[threadIdx.x] = in_w[threadIdx.x];
+    }
+    __syncthreads();
+    const size_t plane = (size_t)T * E, base = (size_t)t * E;
+    const int n4 = E >> 2;
+    float4 u[NV];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int c = threadIdx.x + j * 256;
+        u[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c >= n4) continue;
+        const size_t at = base + (size_t)c * 4;
+        float4 v[HC_MAX_STREAMS];
+#pragma unroll
+        for (int s = 0; s < HC_MAX_STREAMS; ++s)
+            if (s < S) v[s] = *reinterpret_cast<const float4*>(xs + (size_t)s * plane + at);
+        if (y) {
+            const float4 yi = *reinterpret_cast<const float4*>(y + at);
+            float4 nv[HC_MAX_STREAMS];
+#pragma unroll
+            for (int to = 0; to < HC_MAX_STREAMS; ++to) {
+                if (to >= S) continue;
+                float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int s = 0; s < HC_MAX_STREAMS; ++s) {
+                    if (s >= S) continue;
+                    const float m = c_mix[s * S + to];
+                    a.x += m * v[s].x; a.y += m * v[s].y; a.z += m * v[s].z; a.w += m * v[s].w;
+                }
+                const float ow = c_out[to];
+                a.x += ow * yi.x; a.y += ow * yi.y; a.z += ow * yi.z; a.w += ow * yi.w;
+                *reinterpret_cast<float4*>(xs + (size_t)to * plane + at) = a;
+                nv[to] = a;
+            }
+#pragma unroll
+            for (int s = 0; s < HC_MAX_STREAMS; ++s)
+                if (s < S) v[s] = nv[s];
+        }
+        if (h) {
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int s = 0; s < HC_MAX_STREAMS; ++s) {
+                if (s >= S) continue;
+                const float m = c_in[s];
+                a.x += m * v[s].x; a.y += m * v[s].y; a.z += m * v[s].z; a.w += m * v[s].w;
+            }
+            u[j] = a;
+            ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+            if (!norm_w) hc_store4<TO>(h, at, a.x, a.y, a.z, a.w);
+        }
+    }
+    if (!h || !norm_w) return;
+    const float rinv = 1.0f / sqrtf(block_sum_256(ss, part) / (float)E + eps);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int c = threadIdx.x + j * 256;
+        if (c >= n4) continue;
+        const float4 w4 = *reinterpret_cast<const float4*>(norm_w + (size_t)c * 4);
+        hc_store4<TO>(h, base + (size_t)c * 4, u[j].x * rinv * w4.x, u[j].y * rinv * w4.y, u[j].z * rinv * w4.z, u[j].w * rinv * w4.w);
+    }
+}
+
+template <typename TO>
+static void launch_streams_step(float* xs, const float* y, const float* mix, const float* out_w, const float* in_w,
+                                const float* norm_w, TO* h, int T, int E, int S, float eps, hipStream_t stream) {
+    const bool al = ((uintptr_t)xs % 16) == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)norm_w % 16) == 0;
+    if (al && E % 4 == 0 && E <= 4 * 256 * 8) {
+        if (E <= 1024) k_streams_step_v4<TO, 1><<<T, 256, 0, stream>>>(xs, y, mix, out_w, in_w, norm_w, h, T, E, S, eps);
+        else if (E <= 2048) k_streams_step_v4<TO, 2><<<T, 256, 0, stream>>>(xs, y, mix, out_w, in_w, norm_w, h, T, E, S, eps);
+        else if (E <= 4096) k_streams_step_v4<TO, 4><<<T, 256, 0, stream>>>(xs, y, mix, out_w, in_w, norm_w, h, T, E, S, eps);
+        else k_streams_step_v4<TO, 8><<<T, 256, 0, stream>>>(xs, y, mix, out_w, in_w, norm_w, h, T, E, S, eps);
+    } else {
+        k_streams_step<TO><<<T, 256, 0, stream>>>(xs, y, mix, out_w, in_w, norm_w, h, T, E, S, eps);
+    }
+}
+
 extern "C" int xr_streams_step(float* xs, const float* y, const float* mix, const float* out_w, const float* in_w,
                                const float* norm_w, void* h, int T, int E, int S, float eps, int h_dtype, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && E > 0 && S >= 1 && S <= HC_MAX_STREAMS, "streams_step: bad sizes T=%d E=%d S=%d (at most %d streams)", T, E, S,
@@ -188,9 +289,9 @@ extern "C" int xr_streams_step(float* xs, const float* y, const float* mix, cons
     XR_REQUIRE(y || h, "streams_step: nothing to do");
     if (T == 0) return XR_OK;
     if (!h || h_dtype == XR_F32)
-        k_streams_step<float><<<T, 256, 0, stream>>>(xs, y, mix, out_w, in_w, norm_w, (float*)h, T, E, S, eps);
+        launch_streams_step<float>(xs, y, mix, out_w, in_w, norm_w, (float*)h, T, E, S, eps, stream);
     else if (h_dtype == XR_BF16)
-        k_streams_step<bf16_t><<<T, 256, 0, stream>>>(xs, y, mix, out_w, in_w, norm_w, (bf16_t*)h, T, E, S, eps);
+        launch_streams_step<bf16_t>(xs, y, mix, out_w, in_w, norm_w, (bf16_t*)h, T, E, S, eps, stream);
     else { xr_set_error("streams_step: bad dtype %d", h_dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("streams_step");
     return XR_OK;

@@ -82,15 +82,9 @@ class LatentAttention(Mixer):
         self.w_c_norm = tensors[n["dkv_norm"]].float().contiguous()
         self.w_uq = ops.pack_weight(tensors[n["uq"]])
         # Per head: W_uk_h^T [C, D] takes the unrotated query channels into the latent's space,
-        # W_uv_h [Dv, C] the attention's output out of it.  The per-head products read and write
-        # column ranges of wider rows; the matrix-core products take those only where every range
-        # starts on 16 bytes, so the weights are packed for them only then.
-        uk = tensors[n["uk"]].view(H, D, C)
-        uv = tensors[n["uv"]].view(H, Dv, C)
-        aligned = D % 8 == 0 and C % 8 == 0 and self.row % 8 == 0
-        pack = ops.pack_weight if aligned else (lambda w: w)
-        self.w_absorb = [pack(uk[h].t().contiguous()) for h in range(H)]
-        self.w_expand = [pack(uv[h].contiguous()) for h in range(H)]
+        # W_uv_h [Dv, C] the attention's output out of it; each is one launch over all heads.
+        self.w_absorb = tensors[n["uk"]].view(H, D, C).transpose(1, 2).contiguous()      # [H, C, D]
+        self.w_expand = tensors[n["uv"]].view(H, Dv, C).contiguous()                     # [H, Dv, C]
         self.w_out = ops.pack_weight(tensors[n["o"]])
         self.inv_freq = (rotary_inv_freq(self.rot_dims, self.rot_base).to(torch.float32).to(rt.device)
                          if self.rot_dims else None)
@@ -107,8 +101,7 @@ class LatentAttention(Mixer):
         q = torch.empty((T, H * DK), dtype=rt.dtype, device=h.device)
         qn = ops.latent_prepare(q_in, down[:, self.q_rank:], self.w_c_norm, self.eps, q, cache.k, cache.v, ctx, cache.group,
                                 self.inv_freq, H, D, R, C, self.rot_dims, cache.page_size)
-        for hd in range(H):
-            ops.linear(qn[:, hd * D:(hd + 1) * D], self.w_absorb[hd], out=q[:, hd * DK:hd * DK + C])
+        ops.heads_linear(qn, self.w_absorb, q, H, D, DK)
         Dvc = cache.v.shape[2]
         if Dvc == DK and self._matrix_cores():
             o = ops.attention(q, cache.k, cache.v, ctx, cache.group, H, 1, DK, cache.page_size, self.scale, self.window)
@@ -116,8 +109,7 @@ class LatentAttention(Mixer):
             o = ops.attention_pooled(q, cache.k, cache.v, None, None, ctx, cache.group, None, H, 1, DK, Dvc,
                                      cache.page_size, self.scale, self.window or (1 << 30), 0)
         ov = torch.empty((T, H * Dv), dtype=rt.dtype, device=h.device)
-        for hd in range(H):
-            ops.linear(o[:, hd * Dvc:hd * Dvc + C], self.w_expand[hd], out=ov[:, hd * Dv:(hd + 1) * Dv])
+        ops.heads_linear(o, self.w_expand, ov, H, Dvc, Dv)
         return ov
 
     def forward(self, ctx, cache, h):

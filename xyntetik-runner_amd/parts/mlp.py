@@ -147,7 +147,7 @@ class RoutedExperts(FeedForward):
         E, F = self.hidden_size, self.intermediate_size
         r, c, p, u, d = self.names
         # a router of N(0, 0.02) would score all experts alike; a correction that matters is as large as the scores differ
-        specs = {r: ParamSpec((self.num_experts, E), role="vector", init="normal:0.5"),
+        specs = {r: ParamSpec((self.num_experts, E), init="normal:0.5"),
                  c: ParamSpec((self.num_experts,), role="vector", init="normal:0.1")}
         for e in range(self.num_experts):
             specs[f"{p}{e}.{u}"] = ParamSpec((F, E))
@@ -157,7 +157,7 @@ class RoutedExperts(FeedForward):
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         r, c, p, u, d = self.names
-        self.router = tensors[r].float().contiguous()
+        self.router = rt.ops.pack_weight(tensors[r])        # in the rows' dtype: the logits are a 32-bit product of the two
         self.correction = tensors[c].float().contiguous()
         self.w_up = torch.stack([tensors[f"{p}{e}.{u}"] for e in range(self.num_experts)]).contiguous()
         self.w_down = torch.stack([tensors[f"{p}{e}.{d}"] for e in range(self.num_experts)]).contiguous()
