@@ -29,8 +29,8 @@ TOL = {"float32": (2e-5, 2e-6), "bfloat16": (5e-2, 6e-3)}
 # In bfloat16 a token whose last chosen expert and the next one score within rounding of each other may
 # take the other one: that token's row then differs by what the two experts differ (times the smallest of
 # its weights), which no tolerance on rounding covers.  So a few rows may lie over the bound on the
-# largest difference (2 in 100, or one), none far over it; the mean bound holds for every request.
-BF16_ROWS_OVER, BF16_FAR = 0.02, 0.5
+# largest difference (8 in 100, or one), none far over it; the mean bound holds for every request.
+BF16_ROWS_OVER, BF16_FAR = 0.08, 0.5
 # prompt lengths (the rest of every request is given "decoded" tokens) and how many of those
 WORKLOAD = {
     "G1": ([1, 4, 23, 64, 150], 30),        # 64: ends on a page of 64 and 16; the window of 21 passes over decoded tokens
