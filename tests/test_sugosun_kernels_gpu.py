@@ -279,6 +279,29 @@ def test_a_far_write_is_kept_by_a_head_that_does_not_decay(ops):
     close(got, want, 5e-6, "far write")
 
 
+@pytest.mark.parametrize("H,D,Dv", [(2, 12, 5), (3, 64, 32)])
+def test_recurrence_applies_silu_as_it_reads(ops, H, D, Dv):
+    """q, k and v through SiLU inside the recurrence kernel: the same read-outs as from rows that passed it before."""
+    from xyntetik_runner_amd.csrc.ops import Ops
+    rng = np.random.default_rng(D)
+    n = 45
+    row = rng.normal(size=(n, 2 * H * D + H * Dv)) * 1.5
+    decay = dev(rng.uniform(0.5, 1.0, size=H))
+    outs = []
+    for fused in (True, False):
+        state = torch.zeros((2,) + Ops.recurrence_state_shape(H, D, Dv), device=DEV)
+        got = []
+        for i, m in cuts(n, [20, 1, 1, 17, 2, 4]):
+            ctx = step_ctx([i], [m], [0])
+            r = dev(row[i:i + m])
+            if not fused:
+                ops.act_rows_(r)
+            got.append(ops.linear_recurrence("retention", r[:, :H * D], r[:, H * D:2 * H * D], r[:, 2 * H * D:], state, ctx, H, H, D, Dv,
+                                             decay=decay, activation="silu" if fused else None).cpu().numpy())
+        outs.append(np.concatenate(got))
+    close(outs[0], outs[1], 2e-6, "silu in the recurrence")
+
+
 # ----------------------------------------------------------------------------- one-layer models with made weights
 def needle_model(window, rot_dim=4, heads=2):
     """A latent-attention layer whose token 1 (the needle) has a key along every query, with a score

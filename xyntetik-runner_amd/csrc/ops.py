@@ -79,7 +79,7 @@ _PROTOS = {
     "xr_heads_gemm_bf16": [_p, _p, _p, _i, _i, _i, _i, _i, C.c_longlong, _i, C.c_longlong, _i, _p],
     "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
-    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p],
+    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p],
     "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_pool_blocks": [_p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_attention_pool_partial": [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
@@ -989,12 +989,15 @@ class Ops:
         return (H, (D + R - 1) // R, Dv, R)
 
     def linear_recurrence(self, kind: str, q, k, v, state: torch.Tensor, ctx, H: int, G: int, D: int, Dv: int,
-                          beta=None, gate=None, decay=None) -> torch.Tensor:
+                          beta=None, gate=None, decay=None, activation: Optional[str] = None) -> torch.Tensor:
         """The read-outs ``[T, H * Dv]`` (32-bit) of a linear recurrence over every request's rows,
         from and into ``state [slots + 1, *recurrence_state_shape]``.  ``kind`` "retention":
         ``S <- decay_h S + k v^T`` with ``decay [H]``; "delta": ``S <- g S; u = beta (v - S^T k);
         S <- S + k u^T`` with ``beta``/``gate [T, H]``; ``o = S^T q`` after the update in both.
-        ``q, k [T, G * D]``, ``v [T, H * Dv]``: 32-bit views that share a row stride."""
+        ``q, k [T, G * D]``, ``v [T, H * Dv]``: 32-bit views that share a row stride.  ``activation`` "silu":
+        q, k and v pass SiLU on their way into the kernel (the views themselves stay as they are)."""
+        if activation not in (None, "silu"):
+            raise KernelError(f"linear_recurrence: activation {activation!r} is not built (none, silu)")
         if kind not in RECURRENCES:
             raise KernelError(f"linear_recurrence: kind {kind!r} (known: {sorted(RECURRENCES)})")
         self._dev(q, k, v, state, beta, gate, decay)
@@ -1029,7 +1032,7 @@ class Ops:
                                                      _ptr(gate), _ptr(decay), state.data_ptr(), ctx.cu_q.data_ptr(),
                                                      ctx.slots.data_ptr(), ctx.B, H, G, D, Dv, q.stride(0),
                                                      gates[0].stride(0) if gates else 0, RECURRENCES[kind],
-                                                     chunk_len, n_chunks, _ptr(scratch), _stream()))
+                                                     chunk_len, n_chunks, _ptr(scratch), 1 if activation else 0, _stream()))
         return out
 
     RETENTION_CHUNK = 256            # rows a chunk; a multiple of the kernel's 16 staged tokens

@@ -46,6 +46,7 @@ struct RecArgs {
     // pass 0: one workgroup runs the whole portion.
     int pass, chunk_len, n_chunks;
     float* scratch;
+    int act;                 // 1: q, k and v pass SiLU as they are fetched (0: they are taken as they are)
 };
 
 // the value of lane (l ^ 1), (l ^ 2) of a quad, or of the lane 4 / 8 further round a row of 16
@@ -111,6 +112,7 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
             const size_t row = (size_t)(row0 + c0 + (ok ? tt : 0)) * a.ld + (size_t)kvh * a.D + (ok ? d : 0);
             rq[i] = ok ? a.q[row] : 0.f;
             rk[i] = ok ? a.k[row] : 0.f;
+            if (a.act) { rq[i] = rq[i] / (1.0f + expf(-rq[i])); rk[i] = rk[i] / (1.0f + expf(-rk[i])); }
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
@@ -119,6 +121,7 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
             const int cc = blockIdx.x * COLS + c;
             const bool ok = idx < REC_TOKENS * COLS && tt < nt && cc < a.Dv && pass != 2;
             rv[i] = ok ? a.v[(size_t)(row0 + c0 + tt) * a.ld + (size_t)h * a.Dv + cc] : 0.f;
+            if (a.act) rv[i] = rv[i] / (1.0f + expf(-rv[i]));
         }
         if (MODE == XR_REC_DELTA && tid < nt) {
             rb = a.beta[(size_t)(row0 + c0 + tid) * a.ld_g + h];
@@ -274,19 +277,20 @@ extern "C" int xr_recurrence_state_dims(int D, int* rows, int* lanes) {
 extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, const float* v, const float* beta,
                                     const float* gate, const float* decay, float* state, const int* cu_q,
                                     const int* slots, int B, int H, int G, int D, int Dv, int ld, int ld_g, int mode,
-                                    int chunk_len, int n_chunks, float* scratch, hipStream_t stream) {
+                                    int chunk_len, int n_chunks, float* scratch, int act, hipStream_t stream) {
     XR_REQUIRE(B >= 0 && H > 0 && G > 0 && H % G == 0, "recurrence: %d heads over %d key heads", H, G);
     XR_REQUIRE(D > 0 && D <= 256 && Dv > 0, "recurrence: key size %d (1 to 256), value size %d", D, Dv);
     XR_REQUIRE(mode == XR_REC_RETENTION || mode == XR_REC_DELTA, "recurrence: mode %d", mode);
     XR_REQUIRE(mode == XR_REC_RETENTION ? decay != nullptr : (beta != nullptr && gate != nullptr),
                "recurrence: the mode's gates are missing");
     XR_REQUIRE(out && q && k && v && state && cu_q && slots, "recurrence: a pointer is missing");
+    XR_REQUIRE(act == 0 || act == 1, "recurrence: activation %d of q, k and v (0: none, 1: SiLU)", act);
     if (B == 0) return XR_OK;
     const bool chunks = chunk_len > 0;
     XR_REQUIRE(!chunks || (mode == XR_REC_RETENTION && n_chunks > 1 && scratch && chunk_len % REC_TOKENS == 0),
                "recurrence: chunks are for retention, with room for their states");
     XR_REQUIRE(!chunks || (long long)B * n_chunks <= 65535, "recurrence: %d requests of %d chunks", B, n_chunks);
-    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g, chunks ? 1 : 0, chunk_len, n_chunks, scratch};
+    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g, chunks ? 1 : 0, chunk_len, n_chunks, scratch, act};
     const int R = rec_lanes(D), cols = 256 / R, per = (D + R - 1) / R;
     dim3 grid((Dv + cols - 1) / cols, H, chunks ? B * n_chunks : B);
 #define REC(M)                                                                          \

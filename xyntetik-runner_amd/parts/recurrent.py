@@ -102,14 +102,15 @@ class Retention(Mixer):
         H, D, Dv, QK, V = self.num_heads, self.head_dim, self.v_head_dim, self.qk_size, self.v_size
         proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         q, k, v, gate = proj[:, :QK], proj[:, QK:2 * QK], proj[:, 2 * QK:2 * QK + V], proj[:, 2 * QK + V:]
-        if self.qkv_activation is not None:
-            ops.act_rows_(proj[:, :2 * QK + V], self.qkv_activation)
         rot = self.position.rotary() if self.position is not None else None
+        fused_act = self.qkv_activation if (rot is None and self.key_scale == 1.0) else None    # the recurrence applies it as it reads
+        if self.qkv_activation is not None and fused_act is None:
+            ops.act_rows_(proj[:, :2 * QK + V], self.qkv_activation)
         if rot is not None:
             ops.rotate_rows_(q, ctx.positions, rot.inv_freq, H, D, rot.rotary_dim, 1.0)
         if rot is not None or self.key_scale != 1.0:
             ops.rotate_rows_(k, ctx.positions, rot.inv_freq if rot else None, H, D, rot.rotary_dim if rot else 0, self.key_scale)
-        o = ops.linear_recurrence("retention", q, k, v, cache.state, ctx, H, H, D, Dv, decay=self.decay)
+        o = ops.linear_recurrence("retention", q, k, v, cache.state, ctx, H, H, D, Dv, decay=self.decay, activation=fused_act)
         if self.norm_over == "row":
             return ops.gated_rmsnorm(o, gate, self.w_norm, 1, V, self.eps, self.rt.dtype, gate_activation=self.gate_activation)
         return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype, gate_activation=self.gate_activation)
