@@ -116,29 +116,58 @@ __global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs g) {
                     acc[r][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][r], af[u][i], acc[r][i], 0, 0, 0);
     }
     // acc[r][i][e]: output column n0 + r * 16 + 4 * (lane / 16) + e of row i * 16 + lane % 16
+    const bool vec_out = g.ldo % 4 == 0 && g.o_group_stride % 4 == 0 && ((uintptr_t)g.out % 16) == 0;
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         if (!a_ok[i]) continue;
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
             const int n = n0 + r * 16 + lq * 4;
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] = acc[r][i][e];
+                if (g.act == GM_ACT_RELU2) { v[e] = fmaxf(v[e], 0.f); v[e] *= v[e]; }
+            }
+            if (vec_out && n + 3 < g.N) {       // the lane's 4 columns in one store
+                if (g.out_bf16) {
+                    uint2 w2;
+                    w2.x = pack_bf16x2(v[0], v[1]);
+                    w2.y = pack_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<uint2*>((bf16_t*)g.out + orow[i] + n) = w2;
+                } else {
+                    *reinterpret_cast<float4*>((float*)g.out + orow[i] + n) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+                continue;
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 if (n + e >= g.N) continue;
-                float v = acc[r][i][e];
-                if (g.act == GM_ACT_RELU2) { v = fmaxf(v, 0.f); v *= v; }
-                if (g.out_bf16) ((bf16_t*)g.out)[orow[i] + n + e] = f32_to_bf16(v);
-                else ((float*)g.out)[orow[i] + n + e] = v;
+                if (g.out_bf16) ((bf16_t*)g.out)[orow[i] + n + e] = f32_to_bf16(v[e]);
+                else ((float*)g.out)[orow[i] + n + e] = v[e];
             }
         }
     }
 }
 
+// rows_a_tile: 16, 32, 64 or 128 rows of a tile (MT groups of 16); a wave takes 32 weight rows, or 64 where
+// the output is wide enough to fill the chip with such waves (`wide`).
+static int g_grouped_variant = 0;       // measurements only: 0 = choose; 1 = narrow waves; 2 = wide waves
+static int g_grouped_bm = 0;            // measurements only: rows of an experts' tile (0 = choose; 64 or 128)
+extern "C" void xr_grouped_set_variant(int v, int bm) { g_grouped_variant = v; g_grouped_bm = (bm == 64 || bm == 128) ? bm : 0; }
+
 static int launch_grouped(const GroupedArgs& g, int n_tiles_max, int rows_a_tile, hipStream_t stream) {
-    const dim3 grid(n_tiles_max, (g.N + 127) / 128);       // 4 waves x 2 groups of 16 weight rows
+    bool wide = g.N >= 128 && rows_a_tile >= 64;
+    if (g_grouped_variant == 1) wide = false;
+    if (g_grouped_variant == 2) wide = rows_a_tile >= 64;
+    const int per_wg = wide ? 256 : 128;                    // 4 waves x 4 or 2 groups of 16 weight rows
+    const dim3 grid(n_tiles_max, (g.N + per_wg - 1) / per_wg);
     if (rows_a_tile == 16) k_grouped_gemm<1, 2><<<grid, 256, 0, stream>>>(g);
     else if (rows_a_tile == 32) k_grouped_gemm<2, 2><<<grid, 256, 0, stream>>>(g);
-    else k_grouped_gemm<4, 2><<<grid, 256, 0, stream>>>(g);
+    else if (rows_a_tile == 64 && !wide) k_grouped_gemm<4, 2><<<grid, 256, 0, stream>>>(g);
+    else if (rows_a_tile == 64) k_grouped_gemm<4, 4><<<grid, 256, 0, stream>>>(g);
+    else if (!wide) k_grouped_gemm<8, 2><<<grid, 256, 0, stream>>>(g);
+    else k_grouped_gemm<8, 4><<<grid, 256, 0, stream>>>(g);
     return 0;
 }
 
@@ -225,7 +254,8 @@ extern "C" int xr_moe_experts_grouped(float* y, void* z, float* yz, int* scratch
     XR_REQUIRE(grouped_operands_ok(h, w_up, E, ld_h, 0, (long long)F * E) && grouped_operands_ok(z, w_down, F, F, 0, (long long)E * F),
                "moe_experts_grouped: widths and row strides must be multiples of 8 and the operands 16-byte aligned");
     if (T == 0) return XR_OK;
-    const int A = T * top, bm = 64, max_tiles = (A + bm - 1) / bm + n;
+    const int A = T * top, max_tiles = (A + 63) / 64 + n;
+    const int bm = (g_grouped_bm ? g_grouped_bm : (A >= 128 * n ? 128 : 64));     // 128 rows a tile where an expert has that many on average
     int* perm = scratch;
     int* tile_group = perm + A;
     int* tile_start = tile_group + max_tiles;

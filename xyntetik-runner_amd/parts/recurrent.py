@@ -103,7 +103,10 @@ class Retention(Mixer):
         proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         q, k, v, gate = proj[:, :QK], proj[:, QK:2 * QK], proj[:, 2 * QK:2 * QK + V], proj[:, 2 * QK + V:]
         rot = self.position.rotary() if self.position is not None else None
-        fused_act = self.qkv_activation if (rot is None and self.key_scale == 1.0) else None    # the recurrence applies it as it reads
+        # a short portion's recurrence applies the activation as it reads (a kernel less in a decode step); a long
+        # one, which runs in chunks and reads its rows twice, takes rows that passed it before
+        fused_act = self.qkv_activation if (rot is None and self.key_scale == 1.0
+                                            and ctx.max_q_len < ops.RETENTION_CHUNKED_FROM) else None
         if self.qkv_activation is not None and fused_act is None:
             ops.act_rows_(proj[:, :2 * QK + V], self.qkv_activation)
         if rot is not None:
