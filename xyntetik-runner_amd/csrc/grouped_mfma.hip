@@ -157,7 +157,7 @@ static int g_grouped_bm = 0;            // measurements only: rows of an experts
 extern "C" void xr_grouped_set_variant(int v, int bm) { g_grouped_variant = v; g_grouped_bm = (bm == 64 || bm == 128) ? bm : 0; }
 
 static int launch_grouped(const GroupedArgs& g, int n_tiles_max, int rows_a_tile, hipStream_t stream) {
-    bool wide = g.N >= 128 && rows_a_tile >= 64;
+    bool wide = g.N >= 128 && rows_a_tile >= 64 && (long long)n_tiles_max * ((g.N + 255) / 256) >= 256;    // enough such workgroups for the chip
     if (g_grouped_variant == 1) wide = false;
     if (g_grouped_variant == 2) wide = rows_a_tile >= 64;
     const int per_wg = wide ? 256 : 128;                    // 4 waves x 4 or 2 groups of 16 weight rows
@@ -243,7 +243,7 @@ __global__ void k_moe_combine(float* __restrict__ y, const float* __restrict__ y
 }
 
 // The routed experts over many rows: sort, z = relu(up)^2 by expert, yz = down by expert, y = the weighted sum.
-// scratch: ints [A + 3 * max_tiles + 1]; z: bf16 [A, F]; yz: float [A, E].  max_tiles = ceil(A / 64) + n.
+// scratch: ints [A + 3 * (ceil(A / 16) + n) + 1]; z: bf16 [A, F]; yz: float [A, E].
 extern "C" int xr_moe_experts_grouped(float* y, void* z, float* yz, int* scratch, const void* h, const void* w_up,
                                       const void* w_down, const int* idx, const float* wts, int T, int E, int F, int ld_h,
                                       int ld_y, int n, int top, int accumulate, hipStream_t stream) {
@@ -254,8 +254,11 @@ extern "C" int xr_moe_experts_grouped(float* y, void* z, float* yz, int* scratch
     XR_REQUIRE(grouped_operands_ok(h, w_up, E, ld_h, 0, (long long)F * E) && grouped_operands_ok(z, w_down, F, F, 0, (long long)E * F),
                "moe_experts_grouped: widths and row strides must be multiples of 8 and the operands 16-byte aligned");
     if (T == 0) return XR_OK;
-    const int A = T * top, max_tiles = (A + 63) / 64 + n;
-    const int bm = (g_grouped_bm ? g_grouped_bm : (A >= 128 * n ? 128 : 64));     // 128 rows a tile where an expert has that many on average
+    const int A = T * top, avg = A / n;
+    // rows of a tile: what an expert has on average, so that few rows do not idle most of a tile's lanes and the
+    // experts' weights are streamed by many workgroups; 128 where an expert has that many
+    const int bm = g_grouped_bm ? g_grouped_bm : (avg <= 16 ? 16 : avg <= 32 ? 32 : avg < 128 ? 64 : 128);
+    const int max_tiles = (A + bm - 1) / bm + n;           // (at most ceil(A / 16) + n, which is what `scratch` has room for)
     int* perm = scratch;
     int* tile_group = perm + A;
     int* tile_start = tile_group + max_tiles;

@@ -952,7 +952,7 @@ class Ops:
             # many rows: sorted by expert, both products on the matrix cores, then the weighted sum
             A = T * top
             yz = torch.empty((A, E), dtype=torch.float32, device=h.device)
-            scratch = torch.empty((A + 3 * (-(-A // 64) + n) + 1,), dtype=torch.int32, device=h.device)
+            scratch = torch.empty((A + 3 * (-(-A // 16) + n) + 1,), dtype=torch.int32, device=h.device)
             self.lib.check(self.lib.xr_moe_experts_grouped(out.data_ptr(), z.data_ptr(), yz.data_ptr(), scratch.data_ptr(),
                                                            h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(),
                                                            wts.data_ptr(), T, E, F, h.stride(0), out.stride(0), n, top,
