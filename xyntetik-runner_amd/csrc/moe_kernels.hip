@@ -27,9 +27,9 @@ __global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* 
     __syncthreads();
     for (int e = lane; e < n; e += 64) z[e] = expf(z[e] - m) / l;       // the scores
     __syncthreads();
-    // `top` rounds of: the largest score + correction not yet taken, the lower index on a tie.  A score
+    // `top` passes of: the largest score + correction not yet taken, the lower index on a tie.  A score
     // that is no number (the row of a request that does not exist, whose state is whatever memory held)
-    // counts as the smallest, so that every round still finds an expert that exists.
+    // counts as the smallest, so that every pass still finds an expert that exists.
     float total = 0.f;
     int mine = 0;           // lane j keeps the j-th choice
     float mine_s = 0.f;
