@@ -86,7 +86,17 @@ TINY_G4 = {
     ],
 }
 
-CONFIGS = {"G1": (TINY_G1, 21), "G2": (TINY_G2, 22), "G3": (TINY_G3, 23), "G4": (TINY_G4, 24)}
+# a cached row longer than the matrix-core attention takes (272 + 32 channels): the 32-bit attention kernel
+# on bfloat16 storage; one expert in all; a single head
+TINY_G5 = {
+    "architecture": "Sugosun", "vocab": 64, "width": 48, "norm": {"eps": 1e-5}, "streams": 2,
+    "layers": [
+        with_ff(latent(1, 24, 32, 40, 24, 272, 0.1, size=40), moe(16, 1, 1)),
+        with_ff(lightning(2, 8, 24, [0.9, 0.8]), None),
+    ],
+}
+
+CONFIGS = {"G1": (TINY_G1, 21), "G2": (TINY_G2, 22), "G3": (TINY_G3, 23), "G4": (TINY_G4, 24), "G5": (TINY_G5, 25)}
 
 
 def make_model(which: str, folder: str, std: float = 0.12) -> str:

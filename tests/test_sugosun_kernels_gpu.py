@@ -200,7 +200,7 @@ def test_products_head_by_head_in_one_launch(ops, T, G, N, K, aw, ow):
     assert (got[:, ~covered] == 7.0).all()
 
 
-@pytest.mark.parametrize("n,top,E,F,T", [(6, 2, 64, 24, 70), (16, 3, 128, 80, 300), (4, 4, 32, 8, 33)])
+@pytest.mark.parametrize("n,top,E,F,T", [(6, 2, 64, 24, 70), (16, 3, 128, 80, 300), (4, 4, 32, 8, 33), (4, 2, 192, 136, 300), (3, 1, 256, 128, 700)])
 def test_experts_over_many_rows_on_the_matrix_cores(ops, n, top, E, F, T):
     rng = np.random.default_rng(n + T)
     r16 = (lambda a: torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).to(torch.float64).numpy())

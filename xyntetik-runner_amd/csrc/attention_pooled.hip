@@ -12,7 +12,7 @@
 // Dv may differ.  Cache layout: K [page][kv_head][slot][D], V [page][kv_head][Dv][slot].
 #include "common.h"
 
-#define AP_MAX_D 256
+#define AP_MAX_D 512
 
 // ---------------------------------------------------------------- queries out, keys and values into their pages
 template <typename T>

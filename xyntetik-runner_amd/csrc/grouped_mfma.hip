@@ -150,6 +150,138 @@ __global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs g) {
     }
 }
 
+// The same product for tiles of 128 rows where the output is wide: a workgroup computes 128 rows x 128 weight
+// rows, its operands staged in LDS once for all four waves (a wave takes 64 x 64 of them).  K goes in slices
+// of 64: the next slice is fetched into registers (16 bytes a lane and piece, the rows of an expert gathered
+// through `perm`) while the matrix cores work on the one in LDS.  Rows of LDS are 72 elements apart, so the
+// 16 rows a fragment read touches do not all start in one bank.
+#define GL_BM 128
+#define GL_BN 128
+#define GL_KS 64
+#define GL_LD 72
+__global__ __launch_bounds__(256) void k_grouped_gemm_lds(GroupedArgs g) {
+    __shared__ __attribute__((aligned(16))) bf16_t As[GL_BM * GL_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[GL_BN * GL_LD];
+    const int tile = blockIdx.x;
+    int group, row0, rows;
+    if (g.tile_group) {
+        if (tile >= *g.n_tiles) return;
+        group = g.tile_group[tile];
+        row0 = g.tile_start[tile];
+        rows = g.tile_count[tile];
+    } else {
+        group = tile / g.tiles_per_group;
+        row0 = (tile - group * g.tiles_per_group) * GL_BM;
+        rows = g.T - row0 < GL_BM ? g.T - row0 : GL_BM;
+    }
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, lq = lane >> 4;
+    const int wm = wave & 1, wn = wave >> 1;
+    const int nb = blockIdx.y * GL_BN;
+
+    // what this thread copies of a slice: 4 pieces of 16 bytes of the rows and 4 of the weights;
+    // piece j is row (tid / 8) + 32 j, columns (tid % 8) * 8 .. + 8 of the slice
+    const int crow = tid >> 3, ccol = (tid & 7) * 8;
+    const bf16_t* a_src[4];
+    const bf16_t* w_src[4];
+    bool a_on[4], w_on[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int r = crow + 32 * j;
+        a_on[j] = r < rows;
+        const int p = g.perm ? g.perm[row0 + (a_on[j] ? r : 0)] : row0 + (a_on[j] ? r : 0);
+        a_src[j] = g.a + (long long)(g.perm ? p / g.gather_div : p) * g.lda + (long long)group * g.a_group_stride + ccol;
+        const int n = nb + r;
+        w_on[j] = n < g.N;
+        w_src[j] = g.w + (long long)group * g.w_group_stride + (long long)(w_on[j] ? n : 0) * g.K + ccol;
+    }
+    gm_f32x4 acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[r][i] = gm_f32x4{0.f, 0.f, 0.f, 0.f};
+
+    uint4 ra[4], rw[4];
+    auto fetch = [&](int k0) {
+        const bool k_ok = k0 + ccol < g.K;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            ra[j] = make_uint4(0, 0, 0, 0);
+            rw[j] = make_uint4(0, 0, 0, 0);
+            if (k_ok && a_on[j]) ra[j] = *reinterpret_cast<const uint4*>(a_src[j] + k0);
+            if (k_ok && w_on[j]) rw[j] = *reinterpret_cast<const uint4*>(w_src[j] + k0);
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < g.K; k0 += GL_KS) {
+        __syncthreads();                        // the slice before has been read by every wave
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<uint4*>(&As[(crow + 32 * j) * GL_LD + ccol]) = ra[j];
+            *reinterpret_cast<uint4*>(&Ws[(crow + 32 * j) * GL_LD + ccol]) = rw[j];
+        }
+        __syncthreads();
+        if (k0 + GL_KS < g.K) fetch(k0 + GL_KS);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            gm_bf16x8 wf[4], af[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                union { uint4 v; gm_bf16x8 b; } c;
+                c.v = *reinterpret_cast<const uint4*>(&Ws[(wn * 64 + r * 16 + l16) * GL_LD + u * 32 + lq * 8]);
+                wf[r] = c.b;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                union { uint4 v; gm_bf16x8 b; } c;
+                c.v = *reinterpret_cast<const uint4*>(&As[(wm * 64 + i * 16 + l16) * GL_LD + u * 32 + lq * 8]);
+                af[i] = c.b;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[r][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[r], af[i], acc[r][i], 0, 0, 0);
+        }
+    }
+    // acc[r][i][e]: output column nb + wn * 64 + r * 16 + 4 * (lane / 16) + e of the tile's row wm * 64 + i * 16 + lane % 16
+    const bool vec_out = g.ldo % 4 == 0 && g.o_group_stride % 4 == 0 && ((uintptr_t)g.out % 16) == 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r_in_tile = wm * 64 + i * 16 + l16;
+        if (r_in_tile >= rows) continue;
+        const int p = g.perm ? g.perm[row0 + r_in_tile] : row0 + r_in_tile;
+        const long long orow = (long long)p * g.ldo + (long long)group * g.o_group_stride;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = nb + wn * 64 + r * 16 + lq * 4;
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] = acc[r][i][e];
+                if (g.act == GM_ACT_RELU2) { v[e] = fmaxf(v[e], 0.f); v[e] *= v[e]; }
+            }
+            if (vec_out && n + 3 < g.N) {
+                if (g.out_bf16) {
+                    uint2 w2;
+                    w2.x = pack_bf16x2(v[0], v[1]);
+                    w2.y = pack_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<uint2*>((bf16_t*)g.out + orow + n) = w2;
+                } else {
+                    *reinterpret_cast<float4*>((float*)g.out + orow + n) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+                continue;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (n + e >= g.N) continue;
+                if (g.out_bf16) ((bf16_t*)g.out)[orow + n + e] = f32_to_bf16(v[e]);
+                else ((float*)g.out)[orow + n + e] = v[e];
+            }
+        }
+    }
+}
+
 // rows_a_tile: 16, 32, 64 or 128 rows of a tile (MT groups of 16); a wave takes 32 weight rows, or 64 where
 // the output is wide enough to fill the chip with such waves (`wide`).
 static int g_grouped_variant = 0;       // measurements only: 0 = choose; 1 = narrow waves; 2 = wide waves
@@ -160,6 +292,11 @@ static int launch_grouped(const GroupedArgs& g, int n_tiles_max, int rows_a_tile
     bool wide = g.N >= 128 && rows_a_tile >= 64 && (long long)n_tiles_max * ((g.N + 255) / 256) >= 256;    // enough such workgroups for the chip
     if (g_grouped_variant == 1) wide = false;
     if (g_grouped_variant == 2) wide = rows_a_tile >= 64;
+    if (rows_a_tile == 128 && g.N >= 128 && g_grouped_variant != 1 && g_grouped_variant != 2) {     // operands through LDS
+        const dim3 grid_lds(n_tiles_max, (g.N + GL_BN - 1) / GL_BN);
+        k_grouped_gemm_lds<<<grid_lds, 256, 0, stream>>>(g);
+        return 0;
+    }
     const int per_wg = wide ? 256 : 128;                    // 4 waves x 4 or 2 groups of 16 weight rows
     const dim3 grid(n_tiles_max, (g.N + per_wg - 1) / per_wg);
     if (rows_a_tile == 16) k_grouped_gemm<1, 2><<<grid, 256, 0, stream>>>(g);

@@ -26,7 +26,7 @@ import torch
 from .base import KVSpec, Mixer, ParamSpec, register_mixer
 from .rotary import rotary_inv_freq
 
-MAX_ROW = 256       # the attention kernels keep a cached row's channels in registers up to this size
+MAX_ROW = 512       # the 32-bit attention kernel keeps a cached row in registers up to this size (the matrix-core kernels: 256)
 
 
 class LatentAttention(Mixer):
