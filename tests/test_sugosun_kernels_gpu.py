@@ -158,7 +158,7 @@ def test_clamped_gate(ops, limit):
 
 
 # ----------------------------------------------------------------------------- experts
-@pytest.mark.parametrize("n,top,E", [(6, 2, 40), (3, 1, 17), (4, 4, 64), (70, 5, 33)])
+@pytest.mark.parametrize("n,top,E", [(6, 2, 40), (3, 1, 17), (4, 4, 64), (70, 5, 33), (40, 33, 24)])
 def test_routing(ops, n, top, E):
     rng = np.random.default_rng(n * 10 + top)
     T = 50

@@ -10,7 +10,7 @@
 #include "common.h"
 
 #define MOE_MAX_EXPERTS 1024
-#define MOE_MAX_TOP 16
+#define MOE_MAX_TOP 64      // lane j of the routing wave keeps the j-th choice
 
 __global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ logits,
                                                   const float* __restrict__ correction, int ld, int n, int top) {

@@ -131,6 +131,7 @@ class RoutedExperts(FeedForward):
     ``e<i>.down [E, F]``.  Nothing here reads the choice on the host: the kernels find a token's
     experts on the device, so decode steps are recorded like any other."""
     ACTIVATIONS = ("relu2",)
+    MAX_EXPERTS, MAX_TOP = 1024, 64     # MOE_MAX_EXPERTS, MOE_MAX_TOP of csrc/moe_kernels.hip
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, activation: str = "relu2",
                  router_name: str = "router", correction_name: str = "correction", expert_prefix: str = "e",
@@ -139,6 +140,9 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"routed experts: activation {activation!r} is not built (known: {list(self.ACTIVATIONS)})")
         if not (1 <= int(top) <= int(num_experts)):
             raise ValueError(f"routed experts: {top} of {num_experts} experts a token")
+        if int(num_experts) > self.MAX_EXPERTS or int(top) > self.MAX_TOP:       # refused when the model is built, not at its first step
+            raise ValueError(f"routed experts: the kernels take up to {self.MAX_EXPERTS} experts and {self.MAX_TOP} a token, "
+                             f"not {num_experts} and {top}")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.num_experts, self.top = int(num_experts), int(top)
         self.names = (router_name, correction_name, expert_prefix, up_name, down_name)
