@@ -332,14 +332,14 @@ __global__ void k_gate_mul(TO* __restrict__ out, const TI* __restrict__ gu, int 
     int c = (int)(i - t * F);
     float g = ld<TI>(gu, t * ld_gu + c);
     float u = ld<TI>(gu, t * ld_gu + F + c);
-    st<TO>(out, i, gated_value(act, param, g, u));
+    st<TO>(out, i, gate_value<false>(act, param, g, u));
 }
 
 // dtype: of gu; out_dtype: of out (32-bit branches may leave as bfloat16)
 extern "C" int xr_gate_mul(void* out, const void* gu, int T, int F, int ld_gu, int dtype, int out_dtype, int act, float param,
                            hipStream_t stream) {
     XR_REQUIRE(T >= 0 && F > 0 && ld_gu >= 2 * F, "gate_mul: bad sizes T=%d F=%d ld=%d", T, F, ld_gu);
-    XR_REQUIRE(act >= 0 && act < XR_GATE_COUNT, "gate_mul: unknown activation code %d", act);
+    XR_REQUIRE(act >= 0 && act < XR_ACT_COUNT, "gate_mul: unknown activation code %d", act);
     size_t n = (size_t)T * F;
     if (n == 0) return XR_OK;
     unsigned blocks = (unsigned)((n + 255) / 256);

@@ -79,7 +79,8 @@ __host__ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
 // Another activation is another code and another case below; every kernel that applies the
 // gate (the products' epilogues and k_gate_mul) takes the code as an argument.
 #define XR_ACT_SILU 0
-#define XR_ACT_COUNT 1
+#define XR_ACT_CLAMPED_SWISH 1      // takes a number (the limit) and shapes both branches: see gate_value below
+#define XR_ACT_COUNT 2
 #if defined(__HIP_DEVICE_COMPILE__)
 // FAST: with the hardware's 2^x and reciprocal (1 ulp each)
 template <bool FAST> __device__ inline float gate_act(int act, float g) {
@@ -93,24 +94,22 @@ template <bool FAST> __device__ inline float gate_act(int act, float g) {
 template <bool FAST> __host__ __device__ inline float gate_act(int, float g) { return g; }   // the host pass only parses the callers
 #endif
 
-// A gated feed-forward's value from its two branches, for gates that also shape the other branch
-// and take a number of their own.  Codes below XR_ACT_COUNT are act(gate) * up as above (the
-// products' epilogues apply those themselves); the others are applied by k_gate_mul alone.
-// XR_GATE_CLAMPED_SWISH with limit L: g' = min(g, L), u' = clamp(u, -L, L),
-// value = g' sigmoid(1.702 g') (u' + 1).
-#define XR_GATE_CLAMPED_SWISH 1
-#define XR_GATE_COUNT 2
+// A gated feed-forward's value from its two branches and the gate's number: act(gate) * up for the gates
+// above; XR_ACT_CLAMPED_SWISH with limit L shapes both branches: g' = min(g, L), u' = clamp(u, -L, L),
+// value = g' sigmoid(1.702 g') (u' + 1).  The products' epilogues and k_gate_mul all go through this.
 #if defined(__HIP_DEVICE_COMPILE__)
-__device__ inline float gated_value(int act, float param, float g, float u) {
-    if (act == XR_GATE_CLAMPED_SWISH) {
+template <bool FAST> __device__ inline float gate_value(int act, float param, float g, float u) {
+    if (act == XR_ACT_CLAMPED_SWISH) {
         g = fminf(g, param);
         u = fminf(fmaxf(u, -param), param);
-        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+        const float s = FAST ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (-1.702f * 1.44269504f)))
+                             : 1.0f / (1.0f + expf(-1.702f * g));
+        return g * s * (u + 1.0f);
     }
-    return gate_act<false>(act, g) * u;
+    return gate_act<FAST>(act, g) * u;
 }
 #else
-__host__ __device__ inline float gated_value(int, float, float g, float u) { return g * u; }   // the host pass only parses the callers
+template <bool FAST> __host__ __device__ inline float gate_value(int, float, float g, float u) { return g * u; }   // the host pass only parses the callers
 #endif
 
 template <typename T> __device__ inline float ld(const T* p, size_t i);

@@ -69,6 +69,7 @@ struct GemmArgs {
     int out_bf16;      // storage of out
     int epi;
     int act;           // the gate's activation (XR_ACT_*), with EPI_GATED
+    float act_param;   // and its number, for a gate that takes one
     int m_fast;        // tile order of the asynchronous kernel: 1 = consecutive workgroups share a weight tile, 2 = by XCD
     int splits;        // > 1: K is cut into this many ranges, each workgroup writes raw sums to `partial`
     int k_per_split;   // columns per range (a multiple of 64)
@@ -829,7 +830,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const int item, uin
                         const float bg = g.bias && in ? g.bias[oc] : 0.f, bu = g.bias && in ? g.bias[g.N + oc] : 0.f;
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
-                            t[n][e] = gate_act<true>(g.act, acc[i][(jo + n) * 2][e] + bg) * (acc[i][(jo + n) * 2 + 1][e] + bu);
+                            t[n][e] = gate_value<true>(g.act, g.act_param, acc[i][(jo + n) * 2][e] + bg, acc[i][(jo + n) * 2 + 1][e] + bu);
                     }
                     write_tiles<NTO>(stage, t, g.out, g.ldo, g.out_bf16 ? 2 : 0, m0 + wm0 + i * 32, g.M, oc0, g.N, lane);
                 }
@@ -846,7 +847,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, const int item, uin
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     int m = m0 + wm0 + i * 32 + (e / 4) * 8 + lg * 4 + (e % 4);
-                    if (m < g.M) store_out(g, m, oc, gate_act<true>(g.act, acc[i][j][e] + bg) * (acc[i][j + 1][e] + bu));
+                    if (m < g.M) store_out(g, m, oc, gate_value<true>(g.act, g.act_param, acc[i][j][e] + bg, acc[i][j + 1][e] + bu));
                 }
             }
         return;
@@ -938,7 +939,7 @@ __global__ __launch_bounds__(256) void k_gemm_finish(GemmArgs g) {
             for (int i = 0; i < 8; ++i) u += part[i];
         }
         const float bg = g.bias ? g.bias[n] : 0.f, bu = g.bias ? g.bias[g.N + n] : 0.f;
-        store_out(g, m, n, gate_act<false>(g.act, v + bg) * (u + bu));
+        store_out(g, m, n, gate_value<false>(g.act, g.act_param, v + bg, u + bu));
     } else {
         store_out(g, m, n, v + (g.bias ? g.bias[n] : 0.f));
     }
@@ -1227,7 +1228,7 @@ __global__ __launch_bounds__(64 * KSW) void k_gemm_skinny(GemmArgs g) {
         if (SWIGLU) {
             if (ok) {
                 float bg = g.bias ? g.bias[nn] : 0.f, bu = g.bias ? g.bias[g.N + nn] : 0.f;
-                store_out(g, tok, nn, gate_act<false>(g.act, v[0] + bg) * (v[NWT - 1] + bu));
+                store_out(g, tok, nn, gate_value<false>(g.act, g.act_param, v[0] + bg, v[NWT - 1] + bu));
             }
         } else if (g.rope.q_out) {
             // rotated and cached (the partner of a pair is 8 lanes away, or 1)
@@ -1373,7 +1374,7 @@ extern "C" int xr_rope_tile_rows() { return XR_ROPE_TILE_ROWS; }
 // w_packed: the weights are in k_pack_weight's order.
 // workspace (may be null): room for split products, workspace_bytes long; without it K is not split.
 extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float* bias, int M, int N, int K,
-                            int lda, int ldo, int out_dtype, int epi, int act, int variant, int w_packed, float* workspace,
+                            int lda, int ldo, int out_dtype, int epi, int act, float act_param, int variant, int w_packed, float* workspace,
                             size_t workspace_bytes, XrGemmNorm* norm, const XrGemmRope* rope, hipStream_t stream) {
     XR_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     XR_REQUIRE(lda >= K && ldo >= N, "gemm: row strides lda=%d ldo=%d are shorter than K=%d N=%d", lda, ldo, K, N);
@@ -1387,7 +1388,7 @@ extern "C" int xr_gemm_bf16(void* out, const void* a, const void* w, const float
     if (M == 0) return XR_OK;
     GemmArgs g;
     g.a = (const bf16_t*)a; g.w = (const bf16_t*)w; g.w_packed = w_packed ? 1 : 0; g.bias = bias; g.out = out;
-    g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi; g.act = act;
+    g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldo = ldo; g.out_bf16 = out_dtype == XR_BF16; g.epi = epi; g.act = act; g.act_param = act_param;
     g.m_fast = 0; g.splits = 1; g.k_per_split = 0; g.partial = workspace; g.col0 = 0; g.col1 = N;
     g.raw = 0; g.norm_whole = 0; g.vec_out = 0;
     bool want_whole_norm = false;      // a norm after a product of more than 16 rows is asked for and possible

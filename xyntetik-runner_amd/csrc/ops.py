@@ -19,10 +19,9 @@ from . import build as _build
 XR_F32, XR_BF16 = 0, 1
 _CODE = {torch.float32: XR_F32, torch.bfloat16: XR_BF16}
 # activations of a gated feed-forward, by the code the kernels know them under (XR_ACT_* of common.h)
-GATE_ACTIVATIONS = {"silu": 0}
-# gates that also shape the other branch and take a number of their own (XR_GATE_* of common.h): applied by
-# ``gate_mul`` to the 32-bit result of the gate-and-up product, not by the product's epilogue
-SHAPED_GATES = {"clamped_swish": 1}
+GATE_ACTIVATIONS = {"silu": 0, "clamped_swish": 1}
+# gates that take a number of their own (``param``) and shape both branches (``gate_value`` of common.h)
+SHAPED_GATES = {"clamped_swish"}
 NORM_GATES = {"silu": 0, "sigmoid": 1}                  # XR_GATE_SILU / XR_GATE_SIGMOID of sequence_kernels.hip
 
 
@@ -57,7 +56,7 @@ _PROTOS = {
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
     "xr_stream_read": [_p, _sz, _p, _i, _p],
     "xr_gemm_ref": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
-    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _sz, _p, _p, _p],
+    "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p, _sz, _p, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_rope_table": [_p, _p, _p, _i, _i, _f, _p],
     "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
@@ -254,7 +253,7 @@ class Ops:
         F = F2 // 2
         if gu.stride(1) != 1 or F2 % 2:
             raise KernelError("gate_mul input must be [rows, 2F] with unit column stride")
-        code = SHAPED_GATES[activation] if activation in SHAPED_GATES else activation_code(activation)
+        code = activation_code(activation)
         out = torch.empty((T, F), dtype=out_dtype or gu.dtype, device=gu.device)
         self.lib.check(self.lib.xr_gate_mul(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0), dtype_code(gu.dtype),
                                             dtype_code(out.dtype), code, float(param), _stream()))
@@ -391,7 +390,7 @@ class Ops:
         if self._mfma_ok(a, wt):
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, N, K,
                                                  a.stride(0), out.stride(0), dtype_code(out.dtype),
-                                                 1 if accumulate else 0, 0, variant, 1 if packed else 0,
+                                                 1 if accumulate else 0, 0, 0.0, variant, 1 if packed else 0,
                                                  *self._gemm_workspace(a.device),
                                                  C.addressof(norm) if norm is not None else None, None, _stream()))
             return out
@@ -460,11 +459,9 @@ class Ops:
                      variant: int = 0, param: float = 0.0) -> torch.Tensor:
         """``act(a @ w[:F]^T) * (a @ w[F:]^T)`` for ``w [2F, K]`` = gate rows then up rows
         (a matrix, or a ``PackedWeight`` made with ``gated=True``); ``activation`` is one of
-        ``GATE_ACTIVATIONS``, or one of ``SHAPED_GATES`` with its number ``param`` (the product then leaves
-        both branches in 32 bits and ``gate_mul`` makes the value of them)."""
-        if activation in SHAPED_GATES:
-            rows = a.data if isinstance(a, UnscaledRows) else a
-            return self.gate_mul(self.linear(a, w, bias=bias, out_dtype=torch.float32), activation, param, out_dtype=rows.dtype)
+        ``GATE_ACTIVATIONS``, with its number ``param`` for one of ``SHAPED_GATES``.  The matrix-core kernels
+        apply the gate in their epilogue; where they do not serve (float32, sizes they do not take) the
+        product leaves both branches in 32 bits and ``gate_mul`` makes the value of them."""
         act = activation_code(activation)
         packed = isinstance(w, PackedWeight)
         wt = w.data if packed else w
@@ -482,7 +479,7 @@ class Ops:
                 raise KernelError("linear_gated: bias must be float32 [2F]")
             out = torch.empty((M, F), dtype=a.dtype, device=a.device)
             self.lib.check(self.lib.xr_gemm_bf16(out.data_ptr(), a.data_ptr(), wt.data_ptr(), _ptr(bias), M, F, K,
-                                                 a.stride(0), F, dtype_code(out.dtype), 2, act, variant,
+                                                 a.stride(0), F, dtype_code(out.dtype), 2, act, float(param), variant,
                                                  1 if packed else 0, *self._gemm_workspace(a.device),
                                                  C.addressof(norm) if norm is not None else None, None, _stream()))
             return out
@@ -490,7 +487,7 @@ class Ops:
             raise KernelError("linear_gated: rows that still lack their norm's scale need the MFMA kernels")
         if packed:
             raise KernelError("linear_gated: a packed weight needs bfloat16 rows that are 16-byte aligned")
-        return self.gate_mul(self.linear(a, w, bias=bias), activation)
+        return self.gate_mul(self.linear(a, w, bias=bias, out_dtype=torch.float32), activation, param, out_dtype=a.dtype)
 
     def linear_swiglu(self, a: torch.Tensor, w, bias: Optional[torch.Tensor] = None, variant: int = 0) -> torch.Tensor:
         """``linear_gated`` with the SiLU gate."""
@@ -576,7 +573,7 @@ class Ops:
             table = cs_table() if (cs_table is not None and T >= self.ROPE_TILE_ROWS and rot > 0) else None
             rp.cs_table = _ptr(table)
             self.lib.check(self.lib.xr_gemm_bf16(None, rows.data_ptr(), wt.data_ptr(), _ptr(bias), T, w.shape[0],
-                                                 rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0, variant,
+                                                 rows.shape[1], rows.stride(0), w.shape[0], XR_F32, 0, 0, 0.0, variant,
                                                  1 if isinstance(w, PackedWeight) else 0,
                                                  *self._gemm_workspace(rows.device),
                                                  C.addressof(norm) if norm is not None else None,

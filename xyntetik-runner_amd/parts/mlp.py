@@ -1,7 +1,7 @@
 """Gated feed-forward: ``down(act(gate(h)) * up(h))``; act = SiLU is the one activation the
-products' epilogues apply (src/model.c:6399-6407, ``gated_act`` :4451-4452); "clamped_swish"
-with a limit L shapes both branches (``g' = min(g, L)``, ``u' = clamp(u, -L, L)``,
-``g' sigmoid(1.702 g') (u' + 1)``) and is applied to the product's 32-bit result by a kernel of its own.
+reference has (src/model.c:6399-6407, ``gated_act`` :4451-4452); "clamped_swish" with a limit L
+shapes both branches (``g' = min(g, L)``, ``u' = clamp(u, -L, L)``, ``g' sigmoid(1.702 g') (u' + 1)``).  The
+products' epilogues apply either to their 32-bit sums.
 
 ``gate`` and ``up`` are kept as one ``[2F, E]`` matrix so that one product makes both;
 the reference does the reverse for a checkpoint that stores them fused
@@ -30,10 +30,10 @@ class GatedMLP(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", bias: bool = False,
                  gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj",
                  activation_param: float = 0.0, weight_suffix: str = ".weight"):
-        from ..csrc.ops import GATE_ACTIVATIONS, SHAPED_GATES
-        if activation not in GATE_ACTIVATIONS and activation not in SHAPED_GATES:
+        from ..csrc.ops import GATE_ACTIVATIONS
+        if activation not in GATE_ACTIVATIONS:
             raise ValueError(f"gated feed-forward: activation {activation!r} is not built into the kernels "
-                             f"(known: {sorted(GATE_ACTIVATIONS) + sorted(SHAPED_GATES)})")
+                             f"(known: {sorted(GATE_ACTIVATIONS)})")
         self.activation, self.activation_param = activation, float(activation_param)
         self.suffix = weight_suffix
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
@@ -57,12 +57,9 @@ class GatedMLP(FeedForward):
         self.rt = rt
         g, u, d = self.names
         sfx = self.suffix
-        from ..csrc.ops import GATE_ACTIVATIONS
-        # gate rows then up rows, so that one product makes both; in the kernels' own order (a gate
-        # that a kernel of its own applies reads the product's plain result)
+        # gate rows then up rows, so that one product makes both; in the kernels' own order
         self.w_gate_up = rt.ops.pack_weight(
-            torch.cat([tensors[f"{g}{sfx}"], tensors[f"{u}{sfx}"]], dim=0).contiguous(),
-            gated=self.activation in GATE_ACTIVATIONS)
+            torch.cat([tensors[f"{g}{sfx}"], tensors[f"{u}{sfx}"]], dim=0).contiguous(), gated=True)
         self.w_down = rt.ops.pack_weight(tensors[f"{d}{sfx}"])
         if self.bias:
             self.b_gate_up = torch.cat([tensors[f"{g}.bias"], tensors[f"{u}.bias"]]).float().contiguous()
