@@ -157,6 +157,27 @@ def test_clamped_gate(ops, limit):
     close(got.float().cpu(), want, 1e-2, "clamped gate to bfloat16")
 
 
+@pytest.mark.parametrize("T", [3, 40, 700])
+@pytest.mark.parametrize("E,F", [(64, 96), (128, 1024), (40, 20)])
+def test_clamped_gate_in_the_products_epilogue(ops, T, E, F):
+    """The gate-and-up product with the clamped gate, by the skinny, the split and the tile kernels (and,
+    for sizes the matrix cores do not take, the 32-bit product with the gate's own kernel)."""
+    rng = np.random.default_rng(T + F)
+    b16 = lambda x: torch.tensor(x, dtype=torch.float32).to(torch.bfloat16)
+    h, w = b16(rng.normal(size=(T, E))), b16(rng.normal(size=(2 * F, E)) * 0.4)
+    limit = 1.3
+    z = h.double().numpy() @ w.double().numpy().T
+    g, u = np.minimum(z[:, :F], limit), np.clip(z[:, F:], -limit, limit)
+    want = g * G.sigmoid(1.702 * g) * (u + 1.0)
+    assert (z[:, :F] > limit).any() and (np.abs(z[:, F:]) > limit).any()
+    for packed in (False, True):
+        wd = w.to(DEV)
+        got = ops.linear_gated(h.to(DEV), ops.pack_weight(wd, gated=True) if packed else wd, activation="clamped_swish", param=limit)
+        close(got.float().cpu(), want, 1.5e-2, f"packed {packed}")
+    got = ops.linear_gated(h.float().to(DEV), w.float().to(DEV), activation="clamped_swish", param=limit)
+    close(got.cpu(), want, 5e-6, "float32")
+
+
 # ----------------------------------------------------------------------------- experts
 @pytest.mark.parametrize("n,top,E", [(6, 2, 40), (3, 1, 17), (4, 4, 64), (70, 5, 33), (40, 33, 24)])
 def test_routing(ops, n, top, E):
