@@ -1071,7 +1071,8 @@ class Ops:
                                                P, page_size, dtype_code(k_cache.dtype), _stream()))
 
     def attention_pooled(self, q, k_cache, v_cache, pk, pv, ctx, group: int, pool_group: Optional[int], H: int, Hk: int,
-                         D: int, Dv: int, page_size: int, scale: float, size: int, P: int) -> torch.Tensor:
+                         D: int, Dv: int, page_size: int, scale: float, size: int, P: int,
+                         matrix_cores: bool = True) -> torch.Tensor:
         """Attention of every token of the step over the last ``size`` keys of its request and the
         means of the blocks of ``P`` positions that end at least ``size`` positions back (``P`` = 0: none); ``[T, H * Dv]``."""
         self._dev(q, k_cache, v_cache, pk, pv)
@@ -1082,8 +1083,8 @@ class Ops:
         table = ctx.block_table(group)
         ptable = ctx.block_table(pool_group) if P else None
         out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
-        if (self.use_mfma and q.dtype == torch.bfloat16 and D == Dv and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16
-                and H % Hk == 0):
+        if (matrix_cores and self.use_mfma and q.dtype == torch.bfloat16 and D == Dv and D % 16 == 0 and 16 <= D <= 256
+                and page_size >= 16 and H % Hk == 0):
             # The window's keys go to the matrix-core kernels, every row block leaving a partial
             # result; the block means leave theirs in a slot of their own; the kernels' merge adds them.
             lib = self.attention_lib(D)

@@ -107,7 +107,7 @@ class LatentAttention(Mixer):
             o = ops.attention(q, cache.k, cache.v, ctx, cache.group, H, 1, DK, cache.page_size, self.scale, self.window)
         else:
             o = ops.attention_pooled(q, cache.k, cache.v, None, None, ctx, cache.group, None, H, 1, DK, Dvc,
-                                     cache.page_size, self.scale, self.window or (1 << 30), 0)
+                                     cache.page_size, self.scale, self.window or (1 << 30), 0, matrix_cores=False)
         ov = torch.empty((T, H * Dv), dtype=rt.dtype, device=h.device)
         ops.heads_linear(o, self.w_expand, ov, H, Dvc, Dv)
         return ov
