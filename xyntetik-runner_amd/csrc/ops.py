@@ -926,7 +926,10 @@ class Ops:
     def moe_experts(self, h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor,
                     out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
         """``out[t] (+)= sum_j wts[t, j] * w_down[e] @ relu(w_up[e] @ h[t])^2`` with ``e = idx[t, j]``, as 32-bit
-        rows; ``w_up [n, F, E]`` and ``w_down [n, E, F]`` in ``h``'s dtype."""
+        rows; ``w_up [n, F, E]`` and ``w_down [n, E, F]`` in ``h``'s dtype.  A few choices stream the chosen
+        experts' weights, a wave an output column; from ``GROUPED_EXPERTS_FROM`` choices on (bfloat16, widths
+        that are multiples of 8) the rows are sorted by expert on the device, both products run on the matrix
+        cores and a last kernel adds a token's experts up in the order of its choice."""
         self._dev(h, w_up, w_down, idx, wts, out)
         T, E = h.shape
         n, F, _ = w_up.shape
