@@ -156,10 +156,11 @@ __global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs g) {
 // through `perm`) while the matrix cores work on the one in LDS.  Rows of LDS are 72 elements apart, so the
 // 16 rows a fragment read touches do not all start in one bank.
 #define GL_BM 128
-#define GL_BN 128
 #define GL_KS 64
 #define GL_LD 72
+template <int RT>        // groups of 16 weight rows a wave: 4 (128 weight rows a workgroup) or 8 (256)
 __global__ __launch_bounds__(256) void k_grouped_gemm_lds(GroupedArgs g) {
+    constexpr int GL_BN = 32 * RT, WP = RT;       // weight rows a workgroup; 16-byte pieces of them a thread copies a slice
     __shared__ __attribute__((aligned(16))) bf16_t As[GL_BM * GL_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Ws[GL_BN * GL_LD];
     const int tile = blockIdx.x;
@@ -183,32 +184,38 @@ __global__ __launch_bounds__(256) void k_grouped_gemm_lds(GroupedArgs g) {
     // piece j is row (tid / 8) + 32 j, columns (tid % 8) * 8 .. + 8 of the slice
     const int crow = tid >> 3, ccol = (tid & 7) * 8;
     const bf16_t* a_src[4];
-    const bf16_t* w_src[4];
-    bool a_on[4], w_on[4];
+    const bf16_t* w_src[WP];
+    bool a_on[4], w_on[WP];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int r = crow + 32 * j;
         a_on[j] = r < rows;
         const int p = g.perm ? g.perm[row0 + (a_on[j] ? r : 0)] : row0 + (a_on[j] ? r : 0);
         a_src[j] = g.a + (long long)(g.perm ? p / g.gather_div : p) * g.lda + (long long)group * g.a_group_stride + ccol;
-        const int n = nb + r;
+    }
+#pragma unroll
+    for (int j = 0; j < WP; ++j) {
+        const int n = nb + crow + 32 * j;
         w_on[j] = n < g.N;
         w_src[j] = g.w + (long long)group * g.w_group_stride + (long long)(w_on[j] ? n : 0) * g.K + ccol;
     }
-    gm_f32x4 acc[4][4];
+    gm_f32x4 acc[RT][4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+    for (int r = 0; r < RT; ++r)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[r][i] = gm_f32x4{0.f, 0.f, 0.f, 0.f};
 
-    uint4 ra[4], rw[4];
+    uint4 ra[4], rw[WP];
     auto fetch = [&](int k0) {
         const bool k_ok = k0 + ccol < g.K;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             ra[j] = make_uint4(0, 0, 0, 0);
-            rw[j] = make_uint4(0, 0, 0, 0);
             if (k_ok && a_on[j]) ra[j] = *reinterpret_cast<const uint4*>(a_src[j] + k0);
+        }
+#pragma unroll
+        for (int j = 0; j < WP; ++j) {
+            rw[j] = make_uint4(0, 0, 0, 0);
             if (k_ok && w_on[j]) rw[j] = *reinterpret_cast<const uint4*>(w_src[j] + k0);
         }
     };
@@ -216,19 +223,18 @@ __global__ __launch_bounds__(256) void k_grouped_gemm_lds(GroupedArgs g) {
     for (int k0 = 0; k0 < g.K; k0 += GL_KS) {
         __syncthreads();                        // the slice before has been read by every wave
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            *reinterpret_cast<uint4*>(&As[(crow + 32 * j) * GL_LD + ccol]) = ra[j];
-            *reinterpret_cast<uint4*>(&Ws[(crow + 32 * j) * GL_LD + ccol]) = rw[j];
-        }
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(&As[(crow + 32 * j) * GL_LD + ccol]) = ra[j];
+#pragma unroll
+        for (int j = 0; j < WP; ++j) *reinterpret_cast<uint4*>(&Ws[(crow + 32 * j) * GL_LD + ccol]) = rw[j];
         __syncthreads();
         if (k0 + GL_KS < g.K) fetch(k0 + GL_KS);
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            gm_bf16x8 wf[4], af[4];
+            gm_bf16x8 wf[RT], af[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
+            for (int r = 0; r < RT; ++r) {
                 union { uint4 v; gm_bf16x8 b; } c;
-                c.v = *reinterpret_cast<const uint4*>(&Ws[(wn * 64 + r * 16 + l16) * GL_LD + u * 32 + lq * 8]);
+                c.v = *reinterpret_cast<const uint4*>(&Ws[(wn * 16 * RT + r * 16 + l16) * GL_LD + u * 32 + lq * 8]);
                 wf[r] = c.b;
             }
 #pragma unroll
@@ -238,13 +244,13 @@ __global__ __launch_bounds__(256) void k_grouped_gemm_lds(GroupedArgs g) {
                 af[i] = c.b;
             }
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+            for (int r = 0; r < RT; ++r)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     acc[r][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[r], af[i], acc[r][i], 0, 0, 0);
         }
     }
-    // acc[r][i][e]: output column nb + wn * 64 + r * 16 + 4 * (lane / 16) + e of the tile's row wm * 64 + i * 16 + lane % 16
+    // acc[r][i][e]: output column nb + wn * 16 RT + r * 16 + 4 * (lane / 16) + e of the tile's row wm * 64 + i * 16 + lane % 16
     const bool vec_out = g.ldo % 4 == 0 && g.o_group_stride % 4 == 0 && ((uintptr_t)g.out % 16) == 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -253,8 +259,8 @@ __global__ __launch_bounds__(256) void k_grouped_gemm_lds(GroupedArgs g) {
         const int p = g.perm ? g.perm[row0 + r_in_tile] : row0 + r_in_tile;
         const long long orow = (long long)p * g.ldo + (long long)group * g.o_group_stride;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int n = nb + wn * 64 + r * 16 + lq * 4;
+        for (int r = 0; r < RT; ++r) {
+            const int n = nb + wn * 16 * RT + r * 16 + lq * 4;
             float v[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -284,7 +290,7 @@ __global__ __launch_bounds__(256) void k_grouped_gemm_lds(GroupedArgs g) {
 
 // rows_a_tile: 16, 32, 64 or 128 rows of a tile (MT groups of 16); a wave takes 32 weight rows, or 64 where
 // the output is wide enough to fill the chip with such waves (`wide`).
-static int g_grouped_variant = 0;       // measurements only: 0 = choose; 1 = narrow waves; 2 = wide waves
+static int g_grouped_variant = 0;       // measurements only: 0 = choose; 1 = narrow waves; 2 = wide waves; 3, 4 = through LDS, 128 / 256 weight rows
 static int g_grouped_bm = 0;            // measurements only: rows of an experts' tile (0 = choose; 64 or 128)
 extern "C" void xr_grouped_set_variant(int v, int bm) { g_grouped_variant = v; g_grouped_bm = (bm == 64 || bm == 128) ? bm : 0; }
 
@@ -293,8 +299,13 @@ static int launch_grouped(const GroupedArgs& g, int n_tiles_max, int rows_a_tile
     if (g_grouped_variant == 1) wide = false;
     if (g_grouped_variant == 2) wide = rows_a_tile >= 64;
     if (rows_a_tile == 128 && g.N >= 128 && g_grouped_variant != 1 && g_grouped_variant != 2) {     // operands through LDS
-        const dim3 grid_lds(n_tiles_max, (g.N + GL_BN - 1) / GL_BN);
-        k_grouped_gemm_lds<<<grid_lds, 256, 0, stream>>>(g);
+        // (256 weight rows a workgroup, 64 x 128 results a wave, was measured slower: 50 us a product against 35
+        // at 4,096 rows x 1,024 x 2,048; it stays for measurements)
+        const bool big = g_grouped_variant == 4;
+        const int bn = big ? 256 : 128;
+        const dim3 grid_lds(n_tiles_max, (g.N + bn - 1) / bn);
+        if (big) k_grouped_gemm_lds<8><<<grid_lds, 256, 0, stream>>>(g);
+        else k_grouped_gemm_lds<4><<<grid_lds, 256, 0, stream>>>(g);
         return 0;
     }
     const int per_wg = wide ? 256 : 128;                    // 4 waves x 4 or 2 groups of 16 weight rows
