@@ -299,8 +299,8 @@ static int launch_grouped(const GroupedArgs& g, int n_tiles_max, int rows_a_tile
     if (g_grouped_variant == 1) wide = false;
     if (g_grouped_variant == 2) wide = rows_a_tile >= 64;
     if (rows_a_tile == 128 && g.N >= 128 && g_grouped_variant != 1 && g_grouped_variant != 2) {     // operands through LDS
-        // (256 weight rows a workgroup, 64 x 128 results a wave, was measured slower: 50 us a product against 35
-        // at 4,096 rows x 1,024 x 2,048; it stays for measurements)
+        // (256 weight rows a workgroup, 64 x 128 results a wave, was measured slower: sort, both products and
+        // the sum took 176 us against 126 for 4,096 rows over 16 experts of 1,024 x 2,048; it stays for measurements)
         const bool big = g_grouped_variant == 4;
         const int bn = big ? 256 : 128;
         const dim3 grid_lds(n_tiles_max, (g.N + bn - 1) / bn);
