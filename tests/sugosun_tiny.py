@@ -96,7 +96,20 @@ TINY_G5 = {
     ],
 }
 
-CONFIGS = {"G1": (TINY_G1, 21), "G2": (TINY_G2, 22), "G3": (TINY_G3, 23), "G4": (TINY_G4, 24), "G5": (TINY_G5, 25)}
+# the plain residual sum with a pair table; attention without a rotated part, and with two rotated channels
+# of which none turns; a single expert chosen of two
+TINY_G6 = {
+    "architecture": "Sugosun", "vocab": 50, "width": 32, "norm": {"eps": 1e-6},
+    "embedding": {"bigram": {"buckets": 11, "mul_prev": 0, "mul_cur": 1}},
+    "layers": [
+        with_ff(latent(2, 8, 0, 8, 16, 24, 0.3, size=5), moe(8, 2, 1)),
+        with_ff(lightning(2, 4, 4, [0.0, 1.0]), dense(16, 1.0)),
+        with_ff(latent(1, 8, 2, 4, 8, 6, 0.5, dims=0), None),
+    ],
+}
+
+CONFIGS = {"G1": (TINY_G1, 21), "G2": (TINY_G2, 22), "G3": (TINY_G3, 23), "G4": (TINY_G4, 24), "G5": (TINY_G5, 25),
+           "G6": (TINY_G6, 26)}
 
 
 def make_model(which: str, folder: str, std: float = 0.12) -> str:

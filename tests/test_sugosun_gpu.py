@@ -2,7 +2,7 @@
 whole prompts, prompts with their last tokens one by one, portions down to two tokens, mixed
 batches in pools so small that pages and state slots are used again, long decoding through
 recorded steps, and greedy generation through the engine's own entry point and scheduler.
-Four configurations that differ in every size and constant (``sugosun_tiny``)."""
+Six configurations that differ in every size and constant (``sugosun_tiny``)."""
 import io
 import json
 import os
@@ -38,6 +38,7 @@ WORKLOAD = {
     "G3": ([3, 63, 129, 200], 40),          # the window of 64 is a page of 64
     "G4": ([2, 65, 140, 330], 80),          # windows of 70 and 130 pass over pages of 64 in prompts and decoded tokens
     "G5": ([1, 30, 90], 50),
+    "G6": ([1, 2, 17, 40], 12),
 }
 
 
@@ -110,7 +111,7 @@ def steps_for(schedule, reqs, plens, extra):
 
 @pytest.mark.parametrize("schedule", SCHEDULES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which,page_size", [("G1", 16), ("G2", 8), ("G3", 64), ("G4", 64), ("G5", 32)])
+@pytest.mark.parametrize("which,page_size", [("G1", 16), ("G2", 8), ("G3", 64), ("G4", 64), ("G5", 32), ("G6", 4)])
 def test_every_way_of_cutting_gives_the_plain_logits(models, tmp_path, which, page_size, dtype, schedule):
     d, cfg, w, reqs, plens, want = models[which]
     steps = steps_for(schedule, reqs, plens, WORKLOAD[which][1])
